@@ -83,6 +83,8 @@ class ModelSpec:
     position_axes: int = 1
     # (name, rows): a tensor [rows, hidden] of vectors that runs add to the residual stream (`RunStart.vector_row`)
     run_vectors: Optional[tuple] = None
+    # {name: shape}: tensors of the model itself that several layers read (`bind_shared` of their arrangements)
+    shared_tensors: Optional[Dict[str, tuple]] = None
 
     def num_cache_entries(self) -> int:
         ids = [r.cache for r in self.order if r.cache is not None]

@@ -5,7 +5,8 @@
 // latent space after the attention (W_uv,h times the head's result).  The attention itself is the paged kernels'
 // with one key/value head of d >= rank + dr entries.
 //
-//   ilm_latent_prep   from the fused projection rows [q: H (dn + dr) | down: rank + dr]: c = RMS norm of the first
+//   ilm_latent_prep   from the fused projection rows [q: H (dn + dr) | down: rank + dr] (or, without rotated entries, from
+//       rows that hold `down` at any offset: the queries then come from elsewhere): c = RMS norm of the first
 //       rank entries of `down` times a weight; the last dr entries and every head's last dr query entries turned
 //       in pairs (2i, 2i + 1) by pos * freq[i]; key row [c | turned part | zeros] and value column [c | zeros] into
 //       the cache; the turned query parts (and zeros behind them) into the attention's query rows [T, H, d].
@@ -17,12 +18,12 @@ template <typename T, typename TW>
 __global__ void __launch_bounds__(256)
 latent_prep_kernel(const T* __restrict__ rows, T* __restrict__ qx, const int* __restrict__ pos, const float* __restrict__ freq,
                    const TW* __restrict__ w, T* __restrict__ kc, T* __restrict__ vc, const int* __restrict__ slots,
-                   int H, int dn, int dr, int rank, int d, float eps, int page, int stride) {
+                   int H, int dn, int dr, int rank, int d, float eps, int page, int stride, int down_off) {
     extern __shared__ float c[];
     __shared__ float red[4];
     const int t = blockIdx.x, tid = threadIdx.x;
     const T* row = rows + (size_t)t * stride;
-    const T* down = row + (size_t)H * (dn + dr);
+    const T* down = row + down_off;
     float ss = 0.f;
     for (int e = tid; e < rank; e += 256) {
         const float v = to_f32(down[e]);
@@ -70,16 +71,17 @@ latent_prep_kernel(const T* __restrict__ rows, T* __restrict__ qx, const int* __
 
 extern "C" int ilm_latent_prep(const void* rows, void* qx, const void* pos, const void* freq, const void* w, void* kc, void* vc,
                                const void* slots, int T_, int H, int dn, int dr, int rank, int d, float eps, int page,
-                               int stride, int dtype, int w_dt, hipStream_t stream) {
+                               int stride, int down_off, int dtype, int w_dt, hipStream_t stream) {
+    if (down_off < 0) down_off = H * (dn + dr);
     ILM_REQUIRE(T_ > 0 && H > 0 && dn > 0 && dr >= 0 && rank > 0 && page > 0, "latent_prep: bad sizes");
     ILM_REQUIRE(dr % 2 == 0 && d >= rank + dr && rank <= 8192, "latent_prep: %d + %d entries in rows of %d", rank, dr, d);
-    ILM_REQUIRE(stride >= H * (dn + dr) + rank + dr, "latent_prep: rows of %d do not hold the projections", stride);
+    ILM_REQUIRE(stride >= down_off + rank + dr && (dr == 0 || stride >= H * (dn + dr)), "latent_prep: rows of %d do not hold the projections", stride);
     ILM_REQUIRE(dr == 0 || freq != nullptr, "latent_prep: a rotation needs frequencies");
     const size_t shm = (size_t)rank * sizeof(float);
 #define LP_LAUNCH(T__, TW__)                                                                                          \
     latent_prep_kernel<T__, TW__><<<T_, 256, shm, stream>>>((const T__*)rows, (T__*)qx, (const int*)pos, (const float*)freq, \
                                                             (const TW__*)w, (T__*)kc, (T__*)vc, (const int*)slots, H, dn, dr, \
-                                                            rank, d, eps, page, stride)
+                                                            rank, d, eps, page, stride, down_off)
     if (dtype == ILM_DTYPE_F32 && w_dt == ILM_DTYPE_F32) LP_LAUNCH(float, float);
     else if (dtype == ILM_DTYPE_BF16 && w_dt == ILM_DTYPE_BF16) LP_LAUNCH(bf16, bf16);
     else if (dtype == ILM_DTYPE_BF16 && w_dt == ILM_DTYPE_F32) LP_LAUNCH(bf16, float);

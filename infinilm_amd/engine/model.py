@@ -38,6 +38,13 @@ class CausalLM:
         self.run_vectors = None
         if spec.run_vectors is not None:
             self.run_vectors = torch.empty((int(spec.run_vectors[1]), spec.hidden_size), dtype=dtype, device=self.device)
+        # tensors of the model that several layers read (a table of which every layer takes its own columns): made here, loaded
+        # under their own names, handed to every block that asks for them
+        self.shared_tensors = {name: torch.empty(tuple(shape), dtype=dtype, device=self.device)
+                               for name, shape in (spec.shared_tensors or {}).items()}
+        for b in self.blocks:
+            if hasattr(b, "bind_shared"):
+                b.bind_shared(self.shared_tensors)
         self._keeps_embedding = any(r.start is not None and r.start.embedding != 0.0 for r in spec.order)
         # cache entry -> what its writer's mixer needs
         self.cache_needs: List = [None] * spec.num_cache_entries()
@@ -76,6 +83,8 @@ class CausalLM:
             out[join_name(self.spec.final_norm_name, name)] = p
         if self.run_vectors is not None:
             out[self.spec.run_vectors[0]] = Param(self.run_vectors)
+        for name, t in self.shared_tensors.items():
+            out[name] = Param(t)
         if not self.spec.head.always_tied:
             for name, p in self.output_head.named_parameters().items():
                 out[join_name(self.spec.head.name, name)] = p
@@ -95,14 +104,19 @@ class CausalLM:
         return sum(seen.values())
 
     # ---- forward ------------------------------------------------------------------------------
+    def _embed(self, batch) -> torch.Tensor:
+        if getattr(self.embedding, "takes_positions", False):
+            return self.embedding.forward(batch.token_ids, batch.positions)
+        return self.embedding.forward(batch.token_ids)
+
     def forward(self, batch, cache) -> torch.Tensor:
         """float32 logits [len(batch.want_rows), vocab] for the tokens of `batch`."""
-        stream = ResidualStream(self.embedding.forward(batch.token_ids))
+        stream = ResidualStream(self._embed(batch))
         taps = batch.taps
         if taps is not None:
             taps["embed"] = stream.residual.clone()
         # the embedding's output once more for the runs that add it again (the stream itself is summed into in place)
-        first = self.embedding.forward(batch.token_ids) if self._keeps_embedding else None
+        first = self._embed(batch) if self._keeps_embedding else None
         for i, run in enumerate(self.spec.order):
             if run.start is not None:
                 if run.start.embedding != 0.0:
@@ -117,7 +131,7 @@ class CausalLM:
                                    stream.pending_scale)
         if batch.num_wanted == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
-        if stream.more:
+        if stream.more or stream.pending_gate is not None:
             stream.settle()
         if not batch.wants_all_rows:
             last = ResidualStream(kernels.gather_rows(stream.residual, batch.want_rows))

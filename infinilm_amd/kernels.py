@@ -1446,8 +1446,9 @@ def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
 # ---- attention over latent rows -------------------------------------------------------------------
 def latent_prep(rows: torch.Tensor, qx: torch.Tensor, positions: torch.Tensor, freq: Optional[torch.Tensor], weight: torch.Tensor,
                 k_cache: torch.Tensor, v_cache: torch.Tensor, slots: Optional[torch.Tensor], heads: int, dn: int, dr: int, rank: int,
-                d: int, eps: float) -> None:
-    """From fused projection rows [q: heads (dn + dr) | down: rank + dr]: the latent c = RMS norm of down[:rank] times
+                d: int, eps: float, down_offset: int = -1) -> None:
+    """From fused projection rows [q: heads (dn + dr) | down: rank + dr] (`down_offset` >= 0: `down` begins at that entry of a
+    row instead, for queries that are made elsewhere; only without rotated entries): the latent c = RMS norm of down[:rank] times
     `weight`, the last dr entries of `down` and of every query head turned in pairs (2i, 2i + 1) by position x freq[i];
     key row [c | turned part | zeros] and value [c | zeros] into the one-head cache of head size d at `slots`; the
     queries' turned parts (and zeros up to d) into qx [T, heads, d] from entry `rank` on."""
@@ -1457,7 +1458,10 @@ def latent_prep(rows: torch.Tensor, qx: torch.Tensor, positions: torch.Tensor, f
     T = rows.shape[0]
     if tuple(qx.shape) != (T, heads, d) or not qx.is_contiguous() or qx.dtype != rows.dtype:
         raise KernelError(f"the attention's query rows must be contiguous [{T}, {heads}, {d}] of the rows' dtype")
-    if rows.shape[1] != heads * (dn + dr) + rank + dr or weight.shape != (rank,) or not weight.is_contiguous():
+    if down_offset >= 0 and dr:
+        raise KernelError("rows that hold the latent at an offset of their own have no rotated query entries")
+    if (rows.shape[1] != heads * (dn + dr) + rank + dr if down_offset < 0 else rows.shape[1] < down_offset + rank) \
+            or weight.shape != (rank,) or not weight.is_contiguous():
         raise KernelError("rows or norm weight do not fit the latent sizes")
     if dr and (freq is None or freq.dtype != F32 or freq.numel() != dr // 2 or not freq.is_contiguous()):
         raise KernelError(f"frequencies must be float32 [{dr // 2}]")
@@ -1469,7 +1473,7 @@ def latent_prep(rows: torch.Tensor, qx: torch.Tensor, positions: torch.Tensor, f
         page = _check_cache(k_cache, v_cache, 1, d)
     _run("ilm_latent_prep", rows.data_ptr(), qx.data_ptr(), positions.data_ptr(), _ptr(freq), weight.data_ptr(),
          _ptr(k_cache) if slots is not None else None, _ptr(v_cache) if slots is not None else None, _ptr(slots), T, heads, dn, dr,
-         rank, d, float(eps), page, rows.stride(0), _dt(rows), _dt(weight), _stream())
+         rank, d, float(eps), page, rows.stride(0), int(down_offset), _dt(rows), _dt(weight), _stream())
 
 
 HEAD_GEMM_LIBRARY_MIN_ROWS = 33   # rows from which the bfloat16 product per head goes to the vendor library
@@ -1490,4 +1494,190 @@ def head_gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tens
         return out
     _run("ilm_head_gemm", out.data_ptr(), x.data_ptr(), w.data_ptr(), T, N, K, H, x.stride(0), x.stride(1), w.stride(0),
          w.stride(1), w.stride(2), out.stride(0), out.stride(1), _dt(x), _dt(out), _stream())
+    return out
+
+
+# ---- a residual stream whose branches are gated or normed on their way in -----------------------------------------------
+STREAM_PLAIN, STREAM_GATED, STREAM_NORMED = 1, 2, 3
+STREAM_MAX_WIDTH = 12288     # widest row of `stream_update` (the row lies in LDS)
+
+
+def embed_positions(ids: torch.Tensor, positions: torch.Tensor, table: torch.Tensor, position_table: torch.Tensor,
+                    scale: float = 1.0) -> torch.Tensor:
+    """float32 residual rows scale * table[ids] + position_table[positions]."""
+    _dev(ids, positions, table, position_table)
+    _i32(ids, "ids")
+    _i32(positions, "positions")
+    V, H = table.shape
+    if position_table.dim() != 2 or position_table.shape[1] != H or position_table.dtype != table.dtype \
+            or not table.is_contiguous() or not position_table.is_contiguous():
+        raise KernelError("the token table and the position table must be contiguous, of one dtype and one width")
+    T = ids.numel()
+    if positions.numel() != T:
+        raise KernelError("one position a token")
+    out = torch.empty((T, H), dtype=F32, device=table.device)
+    _run("ilm_embed_pos", out.data_ptr(), ids.data_ptr(), positions.data_ptr(), table.data_ptr(), position_table.data_ptr(), T, H, V,
+         position_table.shape[0], float(scale), _dt(table), _stream())
+    return out
+
+
+def stream_update(residual: torch.Tensor, branch: Optional[torch.Tensor] = None, alpha: float = 1.0,
+                  gate: Optional[torch.Tensor] = None, gate_bias: Optional[torch.Tensor] = None,
+                  branch_weight: Optional[torch.Tensor] = None, branch_eps: float = 0.0,
+                  weight: Optional[torch.Tensor] = None, eps: float = 0.0, groups: int = 1,
+                  out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """residual += alpha * f(branch) in place (float32), where f(y) = y, y * sigmoid(gate + gate_bias) with `gate` [T, H], or
+    y / rms(y) * branch_weight (eps inside the root); the branch may come as contiguous float32 parts [P, T, H] that are
+    summed first.  Then, with `out_dtype`: the stream's rows normed in `groups` consecutive equal parts (each by its own root mean
+    square) times `weight`, or without a weight the rows themselves, as out_dtype.  Returns that output or None."""
+    _dev(residual, branch, gate, gate_bias, branch_weight, weight)
+    rows, H = residual.shape
+    if residual.dtype != F32 or not residual.is_contiguous():
+        raise KernelError("the residual stream is a contiguous float32 tensor")
+    if H > STREAM_MAX_WIDTH:
+        raise KernelError(f"rows of {H} are wider than the {STREAM_MAX_WIDTH} this kernel holds")
+    kind, parts, pstride, ystride = 0, 1, 0, H
+    if branch is not None:
+        kind = STREAM_GATED if gate is not None else (STREAM_NORMED if branch_weight is not None else STREAM_PLAIN)
+        if gate is not None and branch_weight is not None:
+            raise KernelError("a branch is gated or normed, not both")
+        y = branch
+        if y.dim() == 3:
+            if not y.is_contiguous() or y.dtype != F32:
+                raise KernelError("parts must be contiguous float32")
+            parts, pstride, y = y.shape[0], y.stride(0), y[0]
+        if tuple(y.shape) != (rows, H) or y.stride(1) != 1:
+            raise KernelError(f"a branch of shape {tuple(branch.shape)} does not fit the stream {tuple(residual.shape)}")
+        ystride = y.stride(0)
+    ws = [t for t in (gate_bias, branch_weight, weight) if t is not None]
+    for t in ws:
+        if tuple(t.shape) != (H,) or not t.is_contiguous() or t.dtype != ws[0].dtype:
+            raise KernelError(f"weights and biases must be contiguous [{H}] of one dtype")
+    if gate is not None and (tuple(gate.shape) != (rows, H) or gate.stride(1) != 1):
+        raise KernelError("the gate's rows must match the stream's")
+    if weight is not None and (groups < 1 or H % groups):
+        raise KernelError(f"rows of {H} do not divide into {groups} groups")
+    if weight is not None and out_dtype is None:
+        raise KernelError("a norm needs an output dtype")
+    out = torch.empty((rows, H), dtype=out_dtype, device=residual.device) if out_dtype is not None else None
+    if kind == 0 and out is None:
+        return None
+    _run("ilm_stream_update", _ptr(out), residual.data_ptr(), _ptr(branch), _ptr(gate), _ptr(gate_bias), _ptr(branch_weight), _ptr(weight),
+         rows, H, int(groups), kind, float(alpha), float(branch_eps), float(eps), _DT[out_dtype] if out is not None else 0,
+         _dt(branch) if branch is not None else 0, _dt(gate) if gate is not None else 0, _dt(ws[0]) if ws else 0, parts, pstride,
+         ystride, gate.stride(0) if gate is not None else 0, _stream())
+    return out
+
+
+def embed_gate(z: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, col0: int) -> torch.Tensor:
+    """g[t, j] = gelu_tanh(z[t, j]) * table[ids[t], col0 + j] for rows z [T, n]."""
+    _dev(z, ids, table)
+    _i32(ids, "ids")
+    _rows(z, "z")
+    T, n = z.shape
+    if table.dim() != 2 or not table.is_contiguous() or table.dtype != z.dtype or ids.numel() != T:
+        raise KernelError("the table must be contiguous and of the rows' dtype, one id a row")
+    out = torch.empty((T, n), dtype=z.dtype, device=z.device)
+    _run("ilm_embed_gate", out.data_ptr(), z.data_ptr(), ids.data_ptr(), table.data_ptr(), T, n, table.shape[1], int(col0), z.stride(0),
+         _dt(z), _stream())
+    return out
+
+
+def softcap_(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """x = cap * tanh(x / cap), in place on a contiguous float32 tensor."""
+    _dev(x)
+    if x.dtype != F32 or not x.is_contiguous():
+        raise KernelError("the capped numbers are a contiguous float32 tensor")
+    if x.numel():
+        _run("ilm_softcap", x.data_ptr(), x.numel(), float(cap), _stream())
+    return x
+
+
+# ---- many small experts of which a token uses a few -----------------------------------------------------------------------
+MOE_TILE_ROWS = 64       # rows of one expert a workgroup of the experts' products takes (ilm_moe_tile_rows())
+MOE_FORCE_PLAIN = os.environ.get("INFINILM_AMD_MOE_PLAIN", "0") == "1"   # 1: the FMA products also in bfloat16
+
+
+class ExpertPlan:
+    """Where every (token, slot) pair of a step lies once the pairs are ordered by expert."""
+    __slots__ = ("ids", "weights", "perm", "inv", "tiles", "n_tiles", "offsets", "max_tiles", "top", "pairs")
+
+
+def moe_route(logits: torch.Tensor, experts: int, top: int) -> ExpertPlan:
+    """From float32 router logits [T, >= experts] (the first `experts` entries of a row count): the `top` experts of every token
+    with sigmoid(logit) as their weights, and the pairs ordered by expert for `moe_gemm`."""
+    _dev(logits)
+    if logits.dtype != F32 or logits.dim() != 2 or logits.stride(1) != 1 or logits.shape[1] < experts:
+        raise KernelError("router logits are float32 rows that hold every expert")
+    T = logits.shape[0]
+    P = T * top
+    plan = ExpertPlan()
+    dev = logits.device
+    plan.top, plan.pairs = int(top), P
+    plan.ids = torch.empty((T, top), dtype=torch.int32, device=dev)
+    plan.weights = torch.empty((T, top), dtype=F32, device=dev)
+    _run("ilm_moe_route", plan.ids.data_ptr(), plan.weights.data_ptr(), logits.data_ptr(), T, int(experts), int(top), logits.stride(0), _stream())
+    plan.max_tiles = min(P, P // MOE_TILE_ROWS + min(experts, P))
+    book = torch.empty((experts + 1 + 2 * P + 3 * plan.max_tiles + 1,), dtype=torch.int32, device=dev)
+    plan.offsets = book[:experts + 1]
+    plan.perm = book[experts + 1:experts + 1 + P]
+    plan.inv = book[experts + 1 + P:experts + 1 + 2 * P]
+    plan.tiles = book[experts + 1 + 2 * P:experts + 1 + 2 * P + 3 * plan.max_tiles]
+    plan.n_tiles = book[-1:]
+    _run("ilm_moe_sort", plan.offsets.data_ptr(), plan.perm.data_ptr(), plan.inv.data_ptr(), plan.tiles.data_ptr(), plan.n_tiles.data_ptr(),
+         plan.ids.data_ptr(), P, int(experts), plan.max_tiles, _stream())
+    return plan
+
+
+def moe_gemm(x: torch.Tensor, w: torch.Tensor, plan: ExpertPlan, glu: bool, limit: float = 0.0, alpha: float = 1.702) -> torch.Tensor:
+    """The experts' products over the ordered pairs.  `glu`: x [T, K] are the tokens' rows, w [E, 2 I, K] holds every expert's
+    gate rows and then its up rows; a pair's row is its token's row times the pair's weight, and the result [pairs, I] is
+    min(gate, limit) * sigmoid(alpha * min(gate, limit)) * (clamp(up, -limit, limit) + 1) in sorted order.  Otherwise x [pairs, K] are rows
+    in sorted order and w [E, N, K]: the result is [pairs, N] in sorted order."""
+    _dev(x, w)
+    _rows(x, "x")
+    E, Nw, K = w.shape
+    if not w.is_contiguous() or w.dtype != x.dtype or x.shape[1] != K or (glu and Nw % 2):
+        raise KernelError(f"experts of shape {tuple(w.shape)} do not fit rows of {tuple(x.shape)}")
+    N = Nw // 2 if glu else Nw
+    if not glu and x.shape[0] != plan.pairs:
+        raise KernelError("rows in sorted order: one a pair")
+    out = torch.empty((plan.pairs, N), dtype=x.dtype, device=x.device)
+    _run("ilm_moe_gemm", out.data_ptr(), N, x.data_ptr(), x.stride(0), plan.perm.data_ptr(), plan.top, plan.weights.data_ptr() if glu else None,
+         w.data_ptr(), Nw * K, K, plan.tiles.data_ptr(), plan.n_tiles.data_ptr(), plan.max_tiles, N, K, int(bool(glu)), float(limit),
+         float(alpha), _dt(x), int(MOE_FORCE_PLAIN), _stream(), label="ilm_moe_gemm (gate/up)" if glu else "ilm_moe_gemm (down)")
+    return out
+
+
+def moe_combine(pair_out: torch.Tensor, plan: ExpertPlan, shared: Optional[torch.Tensor] = None,
+                shared_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y[t] = sum over the token's slots of pair_out[place of (t, slot)] + shared[t] * sigmoid(shared_gate[t]); `shared_gate` is a
+    float32 column (one number a token, any stride)."""
+    _dev(pair_out, shared, shared_gate)
+    _rows(pair_out, "pair_out")
+    P, H = pair_out.shape
+    T = P // plan.top
+    if P != plan.pairs:
+        raise KernelError("one row a pair")
+    sg_stride = 0
+    if shared is not None:
+        if tuple(shared.shape) != (T, H) or not shared.is_contiguous() or shared.dtype != pair_out.dtype:
+            raise KernelError("the shared expert's rows must match the tokens'")
+        if shared_gate is not None:
+            if shared_gate.dtype != F32 or shared_gate.shape[0] != T:
+                raise KernelError("the shared expert's gate is one float32 number a token")
+            sg_stride = shared_gate.stride(0)
+    out = torch.empty((T, H), dtype=pair_out.dtype, device=pair_out.device)
+    _run("ilm_moe_combine", out.data_ptr(), pair_out.data_ptr(), plan.inv.data_ptr(), plan.top, _ptr(shared),
+         _ptr(shared_gate) if shared is not None else None, sg_stride, T, H, pair_out.stride(0), _dt(pair_out), _stream())
+    return out
+
+
+def glu_clamp(gate_up: torch.Tensor, limit: float, alpha: float = 1.702) -> torch.Tensor:
+    """From fused rows [gate | up]: g = min(gate, limit), u = clamp(up, -limit, limit), g * sigmoid(alpha g) * (u + 1)."""
+    _dev(gate_up)
+    _rows(gate_up, "gate_up")
+    T, n = gate_up.shape
+    out = torch.empty((T, n // 2), dtype=gate_up.dtype, device=gate_up.device)
+    _run("ilm_glu_clamp", out.data_ptr(), gate_up.data_ptr(), T, n // 2, gate_up.stride(0), float(limit), float(alpha), _dt(gate_up), _stream())
     return out

@@ -85,6 +85,36 @@ class ResidualStream:
         # norm's output, a copy of the embedding's output, one row for all tokens.  A norm that knows how sums them in its
         # own kernel; anybody else calls `settle()` first
         self.more: list = []
+        # a branch that is still to be multiplied element by element by sigmoid(gate rows + bias) before it is added:
+        # (gate rows [T, hidden], bias [hidden] or None); a norm that knows how does it in its own kernel, `settle()` for
+        # anybody else
+        self.pending_gate = None
+
+    def push_gated(self, branch: torch.Tensor, gate: torch.Tensor, gate_bias, scale: float = 1.0) -> None:
+        """`branch` joins the stream as branch * sigmoid(gate + gate_bias) * scale when the stream is next read."""
+        self.push(branch, scale)
+        self.pending_gate = (gate, gate_bias)
+
+    def rows(self, dtype: torch.dtype) -> torch.Tensor:
+        """Everything that is due summed into the stream, and its rows as `dtype` (float32: the stream's own tensor) for a
+        part that reads the stream itself and not a norm's output."""
+        from .. import kernels
+        if self.more:
+            self.settle()
+        out_dtype = None if dtype == torch.float32 else dtype
+        if self.pending is None:
+            x = kernels.stream_update(self.residual, out_dtype=out_dtype)
+        elif self.pending_gate is not None:
+            x = kernels.stream_update(self.residual, self.pending, self.pending_scale, gate=self.pending_gate[0],
+                                      gate_bias=self.pending_gate[1], out_dtype=out_dtype)
+        elif self.pending_norm is not None and hasattr(self.pending_norm, "weight") and getattr(self.pending_norm, "groups", 1) == 1:
+            x = kernels.stream_update(self.residual, self.pending, self.pending_scale, branch_weight=self.pending_norm.weight,
+                                      branch_eps=self.pending_norm.eps, out_dtype=out_dtype)
+        else:
+            self.settle()
+            x = kernels.stream_update(self.residual, self.pending, self.pending_scale, out_dtype=out_dtype)
+        self.pending, self.pending_scale, self.pending_norm, self.pending_gate = None, 1.0, None, None
+        return self.residual if x is None else x
 
     def push_more(self, addend: torch.Tensor, scale: float = 1.0) -> None:
         """`addend` ([T, hidden], float32 parts [P, T, hidden], or one row [hidden] for every token) times `scale` joins
@@ -108,6 +138,11 @@ class ResidualStream:
         if self.pending_norm is not None:
             norm, self.pending_norm = self.pending_norm, None
             self.pending = norm.apply(self.pending)
+        if self.pending_gate is not None:     # the gated branch goes into the stream now
+            from .. import kernels
+            (gate, bias), self.pending_gate = self.pending_gate, None
+            kernels.stream_update(self.residual, self.pending, self.pending_scale, gate=gate, gate_bias=bias)
+            self.pending, self.pending_scale = None, 1.0
         if self.more:
             from .. import kernels
             more, self.more = self.more, []

@@ -8,6 +8,8 @@ from __future__ import annotations
 
 from typing import Dict
 
+import torch
+
 from ..config.spec import LayerSpec
 from .base import BuildContext, DeferredNorm, Param, ResidualStream, join_name
 from .registry import ARRANGEMENTS, build_feed_forward, build_mixer, build_norm, register_arrangement
@@ -146,6 +148,82 @@ class ParallelResidualBlock:
         stream.push(self.mixer.forward(h, batch, cache_view), self.residual_scale)
         if self.ffn is not None:
             stream.push_more(self.ffn.forward(h, batch), self.residual_scale)
+
+
+@register_arrangement("gated_pre_norm")
+class GatedPreNormBlock:
+    """x += mixer(h) * sigmoid(W_g1 h + b_g1), h = norm1(x); x += ffn(h2) * sigmoid(W_g2 h2 + b_g2), h2 = norm2(x); then, if the
+    layer has one, a side input from the token itself (`side_input.TokenSideInput`).  The gates read what their sublayer
+    reads.  A layer may have no feed-forward (then no norm2 and no second gate), no gates, no side input.  A gated branch is
+    left with the stream together with its gate rows (`ResidualStream.push_gated`): the next norm's kernel multiplies, adds
+    and norms in one pass.  `gate1`, `gate2`: PartSpec("sigmoid_gate", {hidden_size, bias, bias_suffix}); `side`:
+    PartSpec("token_side_input", {...})."""
+
+    def __init__(self, spec: LayerSpec, ctx: BuildContext):
+        from .linear import Linear
+        from .side_input import TokenSideInput
+        self.spec = spec
+        self.slots = tuple(s for s in ("norm1", "mixer", "gate1", "norm2", "ffn", "gate2", "side") if s in spec.parts)
+        if not {"norm1", "mixer"} <= set(self.slots) or (("ffn" in self.slots) != ("norm2" in self.slots)) \
+                or ("gate2" in self.slots and "ffn" not in self.slots):
+            raise ValueError(f"layer {spec.prefix}: a gated layer has norm1, mixer and, with a feed-forward, norm2")
+        self.norm1 = build_norm(spec.parts["norm1"], ctx)
+        self.mixer = build_mixer(spec.parts["mixer"], ctx)
+        self.norm2 = build_norm(spec.parts["norm2"], ctx) if "norm2" in self.slots else None
+        self.ffn = build_feed_forward(spec.parts["ffn"], ctx) if "ffn" in self.slots else None
+        self.gates = {}
+        for slot in ("gate1", "gate2"):
+            if slot in self.slots:
+                p = dict(spec.parts[slot].params)
+                size = int(p["hidden_size"])
+                lin = Linear(size, size, "", False, ctx, suffix="")
+                bias = torch.empty((size,), dtype=ctx.dtype, device=ctx.device) if p.get("bias", True) else None
+                self.gates[slot] = (lin, bias, p.get("bias_suffix", "bias"))
+        self.side = TokenSideInput(ctx=ctx, **spec.parts["side"].params) if "side" in self.slots else None
+        self.residual_scale = float(spec.residual_scale)
+
+    def bind_shared(self, tensors) -> None:
+        if self.side is not None:
+            self.side.bind_shared(tensors)
+
+    def named_parameters(self) -> Dict[str, Param]:
+        out: Dict[str, Param] = {}
+        for slot in self.slots:
+            sub = self.spec.names[slot]
+            if slot in self.gates:
+                lin, bias, suffix = self.gates[slot]
+                for name, p in lin.named_parameters().items():
+                    out[join_name(self.spec.prefix, sub, name)] = p
+                if bias is not None:
+                    out[join_name(self.spec.prefix, sub, suffix)] = Param(bias)
+                continue
+            for name, p in getattr(self, slot).named_parameters().items():
+                out[join_name(self.spec.prefix, sub, name)] = p
+        return out
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    @property
+    def records_mixed_steps(self) -> bool:
+        return bool(getattr(self.mixer, "records_mixed_steps", False)
+                    and (self.ffn is None or getattr(self.ffn, "records_mixed_steps", False)))
+
+    def _push(self, stream: ResidualStream, slot: str, h, y) -> None:
+        if slot in self.gates:
+            lin, bias, _ = self.gates[slot]
+            stream.push_gated(y, lin.forward(h), bias, self.residual_scale)
+        else:
+            stream.push(y, self.residual_scale)
+
+    def forward(self, stream: ResidualStream, batch, cache_view) -> None:
+        h = self.norm1.forward(stream)
+        self._push(stream, "gate1", h, self.mixer.forward(h, batch, cache_view))
+        if self.ffn is not None:
+            h = self.norm2.forward(stream)
+            self._push(stream, "gate2", h, self.ffn.forward(h, batch))
+        if self.side is not None:
+            self.side.forward(stream, batch)
 
 
 def build_block(spec: LayerSpec, ctx: BuildContext):

@@ -51,6 +51,26 @@ class ScaledLookup(Embedding):
         return kernels.embed(token_ids, self.table, self.scale)
 
 
+@register_embedding("positioned_lookup")
+class PositionedLookup(Embedding):
+    """scale * table[token] + position table[position]: a learned row for every position, added unscaled.  `takes_positions`:
+    forward gets the step's positions beside the token ids."""
+    takes_positions = True
+
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float, max_positions: int, ctx: BuildContext,
+                 param_name: str = "weight", position_name: str = "positions"):
+        self.scale = float(scale)
+        self.param_name, self.position_name = param_name, position_name
+        self.table = torch.empty((int(vocab_size), int(hidden_size)), dtype=ctx.dtype, device=ctx.device)
+        self.position_table = torch.empty((int(max_positions), int(hidden_size)), dtype=ctx.dtype, device=ctx.device)
+
+    def named_parameters(self) -> Dict[str, Param]:
+        return {self.param_name: Param(self.table), self.position_name: Param(self.position_table)}
+
+    def forward(self, token_ids: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+        return kernels.embed_positions(token_ids, positions, self.table, self.position_table, self.scale)
+
+
 @register_head("linear")
 class LinearHead(OutputHead):
     """logits = scale * x W^T, float32."""
@@ -73,3 +93,18 @@ class LinearHead(OutputHead):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return kernels.gemm(x, self.weight, None, self.scale, torch.float32)
+
+
+@register_head("capped_linear")
+class CappedLinearHead(LinearHead):
+    """logits = cap * tanh(scale * x W^T / cap), float32."""
+
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float, cap: float, ctx: BuildContext, param_name: str = "weight"):
+        super().__init__(vocab_size, hidden_size, scale, ctx, param_name=param_name)
+        self.cap = float(cap)
+        if self.cap <= 0:
+            raise ValueError(f"a cap on the logits must be positive, got {cap}")
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        z = kernels.gemm(x, self.weight, None, self.scale, torch.float32)
+        return kernels.softcap_(z if z.is_contiguous() else z.contiguous(), self.cap)

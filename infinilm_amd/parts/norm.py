@@ -63,6 +63,43 @@ class RMSNorm(Norm):
         return x
 
 
+@register_norm("group_rmsnorm")
+class GroupRMSNorm(Norm):
+    """RMS norm in `groups` consecutive equal parts of a row: each part is divided by its own sqrt(mean square + eps), the whole
+    row is multiplied by one weight.  Fused with what is due to the residual stream: a plain branch, a branch times
+    sigmoid(gate) (`ResidualStream.push_gated`) or a branch with an RMS norm of its own (`push_normed`) is added in the
+    same kernel (`kernels.stream_update`)."""
+
+    def __init__(self, size: int, eps: float, groups: int, ctx: BuildContext, param_name: str = "weight"):
+        self.size, self.eps, self.groups = int(size), float(eps), int(groups)
+        if self.groups < 1 or self.size % self.groups:
+            raise ValueError(f"rows of {self.size} do not divide into {self.groups} groups")
+        self.dtype = ctx.dtype
+        self.param_name = param_name
+        self.weight = torch.empty((self.size,), dtype=ctx.dtype, device=ctx.device)
+
+    def named_parameters(self) -> Dict[str, Param]:
+        return {self.param_name: Param(self.weight, neutral=1.0)}
+
+    def apply(self, x: torch.Tensor, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+        return kernels.group_norm_gate(x, self.weight, self.eps, self.groups, out_dtype=out_dtype)
+
+    def forward(self, stream: ResidualStream, frag: bool = False):
+        if stream.more:
+            stream.settle()
+        post = stream.pending_norm
+        if post is not None and not (isinstance(post, RMSNorm) and post.weight.dtype == self.weight.dtype):
+            stream.settle()      # a branch norm of another kind: applied by itself
+            post = None
+        gate, bias = stream.pending_gate if stream.pending_gate is not None else (None, None)
+        x = kernels.stream_update(stream.residual, stream.pending, stream.pending_scale, gate=gate, gate_bias=bias,
+                                  branch_weight=post.weight if post is not None else None,
+                                  branch_eps=post.eps if post is not None else 0.0,
+                                  weight=self.weight, eps=self.eps, groups=self.groups, out_dtype=self.dtype)
+        stream.pending, stream.pending_scale, stream.pending_norm, stream.pending_gate = None, 1.0, None, None
+        return x
+
+
 @register_norm("layernorm")
 class LayerNorm(Norm):
     """(x - mean) / sqrt(mean of squared deviations + eps) * weight + bias, fused with the sums that are due to the residual
@@ -83,6 +120,8 @@ class LayerNorm(Norm):
         return out
 
     def forward(self, stream: ResidualStream, frag: bool = False):
+        if stream.pending_gate is not None:
+            stream.settle()
         if stream.pending_norm is not None:
             norm, stream.pending_norm = stream.pending_norm, None
             stream.pending = norm.apply(stream.pending)
