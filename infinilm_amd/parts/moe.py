@@ -27,6 +27,8 @@ from .registry import register_feed_forward
 @register_feed_forward("routed_experts")
 class RoutedExperts(FeedForward):
     records_mixed_steps = True
+    # a look into the routing: a list put here receives every call's chosen experts, int32 [tokens, top] (a copy a call)
+    trace: Optional[list] = None
 
     def __init__(self, hidden_size: int, experts: int, top: int, expert_ff: int, limit: float, ctx: BuildContext,
                  shared_ff: int = 0, shared_limit: Optional[float] = None, alpha: float = 1.702,
@@ -68,6 +70,8 @@ class RoutedExperts(FeedForward):
     def forward(self, x, batch) -> torch.Tensor:
         logits = kernels.gemm(x, self.router.weight, None, 1.0, torch.float32)          # [T, experts (+ 1)]
         plan = kernels.moe_route(logits, self.E, self.top)
+        if RoutedExperts.trace is not None:
+            RoutedExperts.trace.append(plan.ids.clone())
         act = kernels.moe_gemm(x, self.w_gate_up, plan, True, self.limit, self.alpha)   # [pairs, ff], ordered by expert
         pair_out = kernels.moe_gemm(act, self.w_down, plan, False)                      # [pairs, hidden]
         shared = gate = None

@@ -12,9 +12,20 @@ from typing import Dict, List, Optional
 import torch
 
 
-def proj(h: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor] = None) -> torch.Tensor:
-    y = h @ w.T
-    return y if b is None else y + b
+_ROUND = [None]    # the dtype that projections round their operands and results to (`forward(round_to=...)`)
+
+
+def _r(x: torch.Tensor) -> torch.Tensor:
+    return x if _ROUND[0] is None else x.to(_ROUND[0]).to(x.dtype)
+
+
+def proj(h: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor] = None, exact: bool = False) -> torch.Tensor:
+    """W h (+ b).  Under `round_to` the operands and the result are rounded (`exact`: only the operands, for a product whose
+    result stays in 32-bit, as a router's)."""
+    y = _r(h) @ _r(w).T
+    if b is not None:
+        y = y + b
+    return y if exact else _r(y)
 
 
 def unit_rms(x: torch.Tensor, eps: float) -> torch.Tensor:
@@ -81,15 +92,19 @@ def expert(h: torch.Tensor, w: Dict[str, torch.Tensor], pre: str, limit: float) 
     return proj(g * sigmoid(1.702 * g) * (u + 1.0), w[pre + ".down"])
 
 
-def routed_feed_forward(h: torch.Tensor, mlp: dict, w: Dict[str, torch.Tensor], pre: str, chosen: Optional[list] = None) -> torch.Tensor:
+def routed_feed_forward(h: torch.Tensor, mlp: dict, w: Dict[str, torch.Tensor], pre: str, chosen: Optional[list] = None,
+                        forced: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Each token goes to the `top` experts with the largest sigmoid(router) scores; an expert sees the token's row times
     its score (not renormalised) and the outputs are summed.  A shared expert, if any, sees every row and is weighed by
-    one sigmoid number a token."""
+    one sigmoid number a token.  `chosen` receives (the experts picked here [T, top], the scores [T, n]); `forced` [T, top]
+    replaces the pick (for a comparison with a computation that rounds, where two nearly equal scores may change places)."""
     n, top = mlp["router"]["experts"], mlp["router"]["top"]
-    score = sigmoid(proj(h, w[pre + ".router"]))                # [T, n]
+    score = sigmoid(proj(h, w[pre + ".router"], exact=True))    # [T, n]
     pick = torch.topk(score, top, dim=-1).indices               # [T, top]
     if chosen is not None:
-        chosen.append(pick)
+        chosen.append((pick, score))
+    if forced is not None:
+        pick = torch.as_tensor(forced, dtype=torch.long)
     y = torch.zeros_like(h)
     for e in range(n):
         for slot in range(top):
@@ -97,7 +112,7 @@ def routed_feed_forward(h: torch.Tensor, mlp: dict, w: Dict[str, torch.Tensor], 
             if rows.numel():
                 y[rows] += expert(h[rows] * score[rows, e][:, None], w, f"{pre}.e{e}", mlp["expert"]["limit"])
     if mlp.get("shared"):
-        y = y + expert(h, w, pre + ".shared", mlp["shared"]["limit"]) * sigmoid(proj(h, w[pre + ".shared.sg"]))
+        y = y + expert(h, w, pre + ".shared", mlp["shared"]["limit"]) * sigmoid(proj(h, w[pre + ".shared.sg"], exact=True))
     return y
 
 
@@ -118,7 +133,8 @@ def run_order(cfg: dict) -> List[int]:
     return list(range(a)) + list(range(a, b)) * times + list(range(b, n))
 
 
-def layer(cfg: dict, w: Dict[str, torch.Tensor], i: int, x: torch.Tensor, tokens: torch.Tensor) -> torch.Tensor:
+def layer(cfg: dict, w: Dict[str, torch.Tensor], i: int, x: torch.Tensor, tokens: torch.Tensor, chosen: Optional[list] = None,
+          forced: Optional[torch.Tensor] = None) -> torch.Tensor:
     L = cfg["layers"][i]
     eps = cfg["norm"]["eps"]
     h = model_norm(cfg, x, w[f"l{i}.norm1"])
@@ -126,7 +142,7 @@ def layer(cfg: dict, w: Dict[str, torch.Tensor], i: int, x: torch.Tensor, tokens
     x = x + y * sigmoid(proj(h, w[f"l{i}.rg1"], w[f"l{i}.rg1.b"]))
     if L.get("mlp"):
         h = model_norm(cfg, x, w[f"l{i}.norm2"])
-        y = routed_feed_forward(h, L["mlp"], w, f"l{i}.mlp")
+        y = routed_feed_forward(h, L["mlp"], w, f"l{i}.mlp", chosen=chosen, forced=forced)
         x = x + y * sigmoid(proj(h, w[f"l{i}.rg2"], w[f"l{i}.rg2.b"]))
     side = cfg.get("token_side")
     if side:
@@ -134,17 +150,39 @@ def layer(cfg: dict, w: Dict[str, torch.Tensor], i: int, x: torch.Tensor, tokens
     return x
 
 
-def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens, dtype=torch.float64, layers_out: Optional[list] = None) -> torch.Tensor:
-    """Logits [T, vocab] of one sequence."""
+def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens, dtype=torch.float64, round_to=None,
+            layers_out: Optional[list] = None, chosen: Optional[list] = None, forced: Optional[list] = None) -> torch.Tensor:
+    """Logits [T, vocab] of one sequence.  `round_to`: projections take operands and give results rounded to that dtype
+    (what a bfloat16 engine does at its matrix products), everything else stays in `dtype`.  `chosen` receives, for every run
+    of a layer with experts in the order of the runs, (picked experts, scores); `forced`: the picks to use instead, one
+    [T, top] tensor for each such run."""
+    _ROUND[0] = round_to
+    try:
+        return _forward(cfg, w, tokens, dtype, layers_out, chosen, forced)
+    finally:
+        _ROUND[0] = None
+
+
+def greedy(cfg: dict, w: Dict[str, torch.Tensor], prompt, n: int) -> List[int]:
+    """The n tokens greedy decoding appends to `prompt` (the whole sequence is run again for every token)."""
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(int(torch.argmax(forward(cfg, w, toks)[-1])))
+    return toks[len(prompt):]
+
+
+def _forward(cfg, w, tokens, dtype, layers_out, chosen=None, forced=None):
     w = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in w.items()}
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     T = tokens.numel()
     x = w["embed"][tokens] + w["pos"][:T]
+    forced = list(forced) if forced is not None else None
     for i in run_order(cfg):
-        x = layer(cfg, w, i, x, tokens)
+        f = forced.pop(0) if forced is not None and cfg["layers"][i].get("mlp") else None
+        x = layer(cfg, w, i, x, tokens, chosen=chosen, forced=f)
         if layers_out is not None:
             layers_out.append(x.clone())
-    z = proj(model_norm(cfg, x, w["final.norm"]), w["head"])
+    z = proj(model_norm(cfg, x, w["final.norm"]), w["head"], exact=True)
     cap = cfg.get("logit_softcap")
     if cap:
         z = cap * torch.tanh(z / cap)
@@ -203,13 +241,16 @@ def random_weights(cfg: dict, seed: int, store: torch.dtype = torch.bfloat16) ->
 
 def tiny_config(width=64, vocab=97, heads=3, dim=16, vdim=24, kv_rank=32, q_rank=40, window=12, layers=3, experts=4, top=2,
                 ff=48, shared_ff=40, groups=2, side_dim=8, loop=None, softcap=20.0, limit=1.5, max_positions=512,
-                scale=None, mlp_at=None, windows=None) -> dict:
+                scale=None, mlp_at=None, windows=None, mixers=None) -> dict:
     """A small configuration; `mlp_at`: the layers that have a feed-forward (None: all); `windows`: a window a layer
-    (None in the list: that layer sees every earlier token)."""
+    (None in the list: that layer sees every earlier token); `mixers`: a dict a layer of mixer sizes that differ from the
+    common ones."""
     ls = []
     for i in range(layers):
         win = window if windows is None else windows[i]
         mixer = {"dim": dim, "heads": heads, "kv_rank": kv_rank, "q_rank": q_rank, "scale": scale or dim ** -0.5, "vdim": vdim}
+        if mixers is not None and mixers[i]:
+            mixer.update(mixers[i])
         if win:
             mixer["mask"] = {"size": win}
         mlp = None
@@ -227,3 +268,28 @@ def tiny_config(width=64, vocab=97, heads=3, dim=16, vdim=24, kv_rank=32, q_rank
     if loop:
         cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
     return cfg
+
+
+def config_a() -> dict:
+    """Three layers, no loop, two experts a token of four, a shared expert, norms in two parts, every layer alike."""
+    return tiny_config()
+
+
+def config_b() -> dict:
+    """Four layers of which two run twice, one without a feed-forward, one that sees every earlier token, windows of 70, 5
+    and 33, one expert a token of five, no shared expert, norms of the whole row, no cap, a token input of 12 columns, latent
+    rows of 48 (filled up to 64 in the cache), layers of unequal head counts and sizes."""
+    return tiny_config(width=96, vocab=131, heads=4, dim=32, vdim=16, kv_rank=48, q_rank=24, layers=4, experts=5, top=1, ff=40,
+                       shared_ff=0, groups=1, side_dim=12, loop=(1, 3, 2), softcap=None, limit=2.5, mlp_at=[0, 2, 3],
+                       windows=[None, 70, 5, 33], scale=0.2,
+                       mixers=[None, {"heads": 2, "dim": 16, "vdim": 32, "scale": 0.3}, {"kv_rank": 24, "q_rank": 56}, None])
+
+
+def config_c() -> dict:
+    """Three layers of which the first two run three times, eight heads over latent rows of 136 (beyond the matrix-core
+    attention's head sizes), a window longer than most prompts, three experts a token of eight, no token input."""
+    return tiny_config(width=128, vocab=300, heads=8, dim=24, vdim=40, kv_rank=136, q_rank=64, window=200, layers=3, experts=8,
+                       top=3, ff=72, shared_ff=24, groups=4, side_dim=0, loop=(0, 2, 3), softcap=8.0, limit=1.0)
+
+
+CONFIGS = {"A": config_a, "B": config_b, "C": config_c}
