@@ -54,7 +54,7 @@ def main() -> int:
                     help="instead of the default workload: prefill and decode throughput of the Kekevik design beside MiniCPM4 "
                          "at equal layer sizes (random weights), with the time and the roofline share of every kernel")
     ap.add_argument("--design-shapes", default="1024,4096", help="widths to compare with --designs")
-    ap.add_argument("--design", default="kekevik", choices=["kekevik", "pugavik"],
+    ap.add_argument("--design", default="kekevik", choices=["kekevik", "pugavik", "patadra"],
                     help="the design that --designs puts beside MiniCPM4")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -94,7 +94,7 @@ def compare_designs(args) -> dict:
     from infinilm_amd.sampling import Sampler, SamplingParams
     from infinilm_amd.weights import fill_random_
     sys.path.insert(0, os.path.join(ROOT, "examples"))
-    from shapes import kekevik_shape, pugavik_shape
+    from shapes import kekevik_shape, patadra_shape, pugavik_shape
 
     layers = 8 if args.layers == 32 else args.layers
     T, ctx, ps = args.prefill_tokens, min(args.context, 2048), args.page_size
@@ -110,7 +110,8 @@ def compare_designs(args) -> dict:
                          "num_hidden_layers": layers, "hidden_size": width, "num_attention_heads": heads, "num_key_value_heads": kv,
                          "head_dim": d, "intermediate_size": 4 * width, "vocab_size": V, "max_position_embeddings": 32768,
                          "rms_norm_eps": 1e-6, "tie_word_embeddings": True},
-            design: (kekevik_shape if design == "kekevik" else pugavik_shape)(width, heads, d, kv, layers, V, 6 * width)}
+            design: patadra_shape(width, heads, d, layers, V) if design == "patadra" else
+            (kekevik_shape if design == "kekevik" else pugavik_shape)(width, heads, d, kv, layers, V, 6 * width)}
         rec = {}
         for name, cfg in cfgs.items():
             model = build_model(cfg, "bfloat16", "cuda:0")
@@ -184,13 +185,37 @@ def compare_designs(args) -> dict:
                     share = {}
                     state = heads * d * d * 4          # a head's state x heads (key size = value size = state entries = d here)
                     kvb = 2 * kv * d * 2               # cached bytes a token
-                    if name != "pugavik" and us(rep_d, "ilm_decay_scan"):
+                    if name == "patadra":
+                        m0 = cfg["layers"][0]
+                        E, top, ff, win = m0["mlp"]["router"]["experts"], m0["mlp"]["router"]["top"], m0["mlp"]["expert"]["ff"], m0["mixer"]["mask"]["size"]
+                        gu, dn = "ilm_moe_gemm (gate/up)", "ilm_moe_gemm (down)"
+                        if us(rep_p, gu):
+                            share["experts' gate/up product prefill (flops / bf16 matrix peak)"] = round(2.0 * T * top * 2 * ff * Hs / us(rep_p, gu) / FLOP_PEAK["bf16"], 4)
+                            share["experts' down product prefill (flops / bf16 matrix peak)"] = round(2.0 * T * top * ff * Hs / us(rep_p, dn) / FLOP_PEAK["bf16"], 4)
+                            hit = min(E, 64 * top)
+                            share["experts' gate/up product decode (weights of the experts hit read / HBM peak)"] = round(hit * 2 * ff * Hs * 2 / us(rep_d, gu) / HBM_PEAK, 4)
+                            share["experts' down product decode (weights of the experts hit read / HBM peak)"] = round(hit * ff * Hs * 2 / us(rep_d, dn) / HBM_PEAK, 4)
+                        lat = "ilm_attn_headmix_mfma"   # (one cached row of d entries a token, read as key and as value)
+                        if us(rep_d, lat):
+                            share["latent attention decode (window's cache read / HBM peak)"] = round(64 * min(ctx, win) * 2 * d * 2 / us(rep_d, lat) / HBM_PEAK, 4)
+                        if us(rep_p, lat):
+                            pairs = sum(min(i + 1, win) for i in range(T))
+                            share["latent attention prefill (4 d flops a visible key and head / bf16 matrix peak)"] = round(
+                                4.0 * d * pairs * heads / us(rep_p, lat) / FLOP_PEAK["bf16"], 4)
+                        if us(rep_p, "ilm_stream_update"):
+                            share["stream_update prefill (stream read + written, branch and gate read, rows written / HBM peak)"] = round(
+                                T * Hs * (4 + 4 + 2 + 2 + 2) / us(rep_p, "ilm_stream_update") / HBM_PEAK, 4)
+                    if name == "minicpm4" and us(rep_p, "library_gemm"):
+                        flops = 2.0 * T * Hs * ((heads + 2 * kv) * d + heads * d + 3 * cfg["intermediate_size"]) * layers
+                        share["library products prefill, all of a step (flops / bf16 matrix peak)"] = round(
+                            flops / (rep_p["library_gemm"]["total_ms"] * 1e-3 / 2) / FLOP_PEAK["bf16"], 4)
+                    if name not in ("pugavik", "patadra") and us(rep_d, "ilm_decay_scan"):
                         share["decay_scan decode (state read + written / HBM peak)"] = round(64 * 2 * state / us(rep_d, "ilm_decay_scan") / HBM_PEAK, 4)
                         share["decay_scan prefill (4 dk dv flops a token and head / float32 vector peak)"] = round(
                             4.0 * T * heads * d * d / us(rep_p, "ilm_decay_scan") / FLOP_PEAK["fp32"], 4)
-                    if name != "pugavik" and us(rep_d, "ilm_attn_mfma"):
+                    if name not in ("pugavik", "patadra") and us(rep_d, "ilm_attn_mfma"):
                         share["attention decode (cache read / HBM peak)"] = round(64 * ctx * kvb / us(rep_d, "ilm_attn_mfma") / HBM_PEAK, 4)
-                    if name != "pugavik" and us(rep_p, "ilm_attn_tile"):
+                    if name not in ("pugavik", "patadra") and us(rep_p, "ilm_attn_tile"):
                         share["attention prefill (4 d flops a visible key and head / bf16 matrix peak)"] = round(
                             4.0 * T * T / 2 * heads * d / us(rep_p, "ilm_attn_tile") / FLOP_PEAK["bf16"], 4)
                     if name == "pugavik":

@@ -13,8 +13,11 @@ def _factors(n: int, seed: int):
 
 
 def shape_config(name: str, layers: int = 0) -> dict:
-    """`name`: "8b", "0.5b", "2b" (MiniCPM4 family), "kekevik-<width>" or "pugavik-<width>" (those designs at that width,
-    8 layers unless told otherwise); `layers` > 0 overrides the number of layers."""
+    """`name`: "8b", "0.5b", "2b" (MiniCPM4 family), "kekevik-<width>", "pugavik-<width>" or "patadra-<width>" (those designs at
+    that width, 8 layers unless told otherwise); `layers` > 0 overrides the number of layers."""
+    if name.startswith("patadra-"):
+        width = int(name.split("-")[1])
+        return patadra_shape(width, width // 128, 128, layers or 8, 32768)
     if name.startswith("kekevik-"):
         width = int(name.split("-")[1])
         return kekevik_shape(width, width // 128, 128, 2, layers or 8, 32768, 6 * width)
@@ -79,6 +82,24 @@ def pugavik_shape(width: int, heads: int, head_dim: int, kv_heads: int, layers: 
     kinds = [("latent_attention", latent), ("attention", att), ("gla", gla)]
     cfg = {"architecture": "Pugavik", "vocab": vocab, "width": width, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5},
            "layers": [{"type": kinds[i % 3][0], "mixer": kinds[i % 3][1], "mlp": {"kind": "dense", "ff": ff}} for i in range(layers)]}
+    if loop:
+        cfg["loop"] = dict(loop)
+    return cfg
+
+
+def patadra_shape(width: int, heads: int, head_dim: int, layers: int, vocab: int, experts: int = 16, top: int = 2, window: int = 1024,
+                  max_positions: int = 4096, loop: dict = None) -> dict:
+    """A Patadra configuration with the layer sizes of a transformer of this width: `heads` heads with queries, keys and values
+    of `head_dim`, latent rows of `head_dim` (one cached row a token), queries through a row of a quarter of the width; `experts`
+    experts with `width` inner units each, of which a token uses `top`, and a shared expert of the same size (three times the
+    width of inner units at work for a token); norms in four parts, a token input of 256 columns a layer, capped logits."""
+    mixer = {"heads": heads, "dim": head_dim, "vdim": head_dim, "kv_rank": head_dim, "q_rank": width // 4, "scale": head_dim ** -0.5,
+             "mask": {"size": window}}
+    mlp = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": width, "limit": 7.0},
+           "shared": {"ff": width, "limit": 7.0}}
+    cfg = {"architecture": "Patadra", "vocab": vocab, "width": width, "max_positions": max_positions, "norm": {"eps": 1e-5, "groups": 4},
+           "logit_softcap": 30.0, "token_side": {"dim": 256},
+           "layers": [{"type": "latent_attention", "mixer": dict(mixer), "mlp": dict(mlp)} for _ in range(layers)]}
     if loop:
         cfg["loop"] = dict(loop)
     return cfg

@@ -547,9 +547,18 @@ def test_random_configurations_in_bfloat16(seed, tmp_path):
     for rid, t in (("a", ta), ("b", tb)):
         picks = drv.request_picks(rid, len(t)) if any(layer["mlp"] for layer in cfg["layers"]) else None
         want = P.forward(cfg, W, t, forced=picks)
-        tol = max(TOL["bfloat16"], 2.0 * rel_err(P.forward(cfg, W, t, forced=picks, round_to=BF), want))
-        err = rel_err(drv.request_logits(rid, len(t)), want)
-        assert err < tol, f"seed {seed} request {rid}: {err:.3e} (bound {tol:.3e}); {json.dumps(cfg)}"
+        lossy = P.forward(cfg, W, t, forced=picks, round_to=BF)
+        # A branch that is divided by its own root mean square (the token input, a few numbers wide here) multiplies a rounding
+        # error many times at the positions where that root mean square happens to be small, so single positions err several
+        # times more than most, in the plain implementation with rounded products too, at positions of its own.  The engine is
+        # held to that implementation's errors: at most positions (the median) closely, at the worst position loosely.
+        top = max(1.0, float(want.abs().max()))
+        e = (drv.request_logits(rid, len(t)).double() - want).abs().amax(-1) / top
+        l = (lossy - want).abs().amax(-1) / top
+        what = f"seed {seed} request {rid}: median {float(e.median()):.3e} (plain, rounded: {float(l.median()):.3e}), " \
+               f"worst {float(e.max()):.3e} ({float(l.max()):.3e}); {json.dumps(cfg)}"
+        assert float(e.median()) < max(TOL["bfloat16"] / 8, 1.5 * float(l.median())), what
+        assert float(e.max()) < max(TOL["bfloat16"], 5.0 * float(l.max())), what
 
 
 # ---- the entry point and its scheduler ------------------------------------------------------------------------------------
