@@ -21,6 +21,7 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 #define MOE_MAX_E 1024
 #define MOE_TM 64
+#define MOE_BM 128  // rows of a tile of the many-rows kernel
 #define MOE_TN 64
 #define MOE_KS 64
 #define MOE_LD (MOE_KS + 8)   // bf16 elements a row of a tile in LDS (144 bytes)
@@ -79,7 +80,7 @@ extern "C" int ilm_moe_route(void* ids, void* wts, const void* z, int T_, int E,
 // ---- ordering by expert --------------------------------------------------------------------------------------------
 __global__ void __launch_bounds__(1024)
 moe_sort_kernel(int* __restrict__ offsets, int* __restrict__ perm, int* __restrict__ inv, int* __restrict__ tiles, int* __restrict__ n_tiles,
-                const int* __restrict__ ids, int P, int E, int max_tiles) {
+                const int* __restrict__ ids, int P, int E, int max_tiles, int tile_rows) {
     __shared__ int cnt[MOE_MAX_E], cur[MOE_MAX_E], tbase[MOE_MAX_E];
     const int tid = threadIdx.x;
     for (int e = tid; e < E; e += 1024) cnt[e] = 0;
@@ -96,7 +97,7 @@ moe_sort_kernel(int* __restrict__ offsets, int* __restrict__ perm, int* __restri
             cur[e] = off;
             tbase[e] = tb;
             off += cnt[e];
-            tb += (cnt[e] + MOE_TM - 1) / MOE_TM;
+            tb += (cnt[e] + tile_rows - 1) / tile_rows;
         }
         offsets[E] = off;
         *n_tiles = tb < max_tiles ? tb : max_tiles;
@@ -104,10 +105,10 @@ moe_sort_kernel(int* __restrict__ offsets, int* __restrict__ perm, int* __restri
     __syncthreads();
     for (int e = tid; e < E; e += 1024) {
         const int n = cnt[e], base = cur[e];
-        for (int i = 0, tb = tbase[e]; i < n && tb < max_tiles; i += MOE_TM, ++tb) {
+        for (int i = 0, tb = tbase[e]; i < n && tb < max_tiles; i += tile_rows, ++tb) {
             tiles[3 * tb] = e;
             tiles[3 * tb + 1] = base + i;
-            tiles[3 * tb + 2] = n - i < MOE_TM ? n - i : MOE_TM;
+            tiles[3 * tb + 2] = n - i < tile_rows ? n - i : tile_rows;
         }
     }
     __syncthreads();
@@ -124,11 +125,12 @@ moe_sort_kernel(int* __restrict__ offsets, int* __restrict__ perm, int* __restri
 extern "C" int ilm_moe_tile_rows() { return MOE_TM; }
 
 extern "C" int ilm_moe_sort(void* offsets, void* perm, void* inv, void* tiles, void* n_tiles, const void* ids, int P, int E,
-                            int max_tiles, hipStream_t stream) {
+                            int max_tiles, int tile_rows, hipStream_t stream) {
     ILM_REQUIRE(P > 0 && E > 0 && E <= MOE_MAX_E, "moe_sort: %d pairs, %d experts (at most %d)", P, E, MOE_MAX_E);
-    const int need = P / MOE_TM + (E < P ? E : P);
+    ILM_REQUIRE(tile_rows == MOE_TM || tile_rows == MOE_BM, "moe_sort: tiles of %d rows (%d or %d)", tile_rows, MOE_TM, MOE_BM);
+    const int need = P / tile_rows + (E < P ? E : P);
     ILM_REQUIRE(max_tiles >= (need < P ? need : P), "moe_sort: %d tiles do not hold %d pairs of %d experts", max_tiles, P, E);
-    moe_sort_kernel<<<1, 1024, 0, stream>>>((int*)offsets, (int*)perm, (int*)inv, (int*)tiles, (int*)n_tiles, (const int*)ids, P, E, max_tiles);
+    moe_sort_kernel<<<1, 1024, 0, stream>>>((int*)offsets, (int*)perm, (int*)inv, (int*)tiles, (int*)n_tiles, (const int*)ids, P, E, max_tiles, tile_rows);
     ILM_LAUNCH_CHECK("moe_sort");
     return 0;
 }
@@ -267,6 +269,134 @@ moe_gemm_mfma_kernel(bf16* __restrict__ out, int ld_out, const bf16* __restrict_
     }
 }
 
+
+// bfloat16 on the matrix cores, many rows an expert.  Block: 4 waves; tile: up to 128 rows of one expert x 128 rows of W (GLU: the
+// gate rows and the up rows of 64 outputs; else 128 outputs); wave (wm, wn) owns 64 rows x 64 rows of W (GLU: gate and up of
+// 32 outputs, so the activation has both in one thread): 16 products for 8 fragment reads a k-step.  blockIdx.x walks the row
+// tiles, so the tiles of one expert, which read the same rows of W, run side by side.
+template <bool GLU>
+__global__ void __launch_bounds__(256)
+moe_gemm_mfma128_kernel(bf16* __restrict__ out, int ld_out, const bf16* __restrict__ X, int ldx, const int* __restrict__ perm, int top,
+                        const float* __restrict__ pair_w, const bf16* __restrict__ W, size_t w_expert, int ldw, const int* __restrict__ tiles,
+                        const int* __restrict__ n_tiles, int N, int K, float limit, float alpha) {
+    constexpr int TN = GLU ? 64 : 128;
+    __shared__ __attribute__((aligned(16))) bf16 xs[MOE_BM * MOE_LD];
+    __shared__ __attribute__((aligned(16))) bf16 ws[128 * MOE_LD];
+    __shared__ int src_row[MOE_BM];
+    __shared__ float src_w[MOE_BM];
+    const int tile = blockIdx.x;
+    if (tile >= *n_tiles) return;
+    const int e = tiles[3 * tile], place0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
+    const int n0 = blockIdx.y * TN, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, wm = wave >> 1, wn = wave & 1;
+    if (tid < MOE_BM) {
+        int row = -1;
+        float w = 1.0f;
+        if (tid < rows) {
+            if (GLU) {
+                const int pair = perm != nullptr ? perm[place0 + tid] : place0 + tid;
+                row = pair / top;
+                if (pair_w != nullptr) w = pair_w[pair];
+            } else {
+                row = place0 + tid;
+            }
+        }
+        src_row[tid] = row;
+        src_w[tid] = w;
+    }
+    __syncthreads();
+    const bf16* We = W + (size_t)e * w_expert;
+    const int lr = tid >> 3, lc = tid & 7;        // this thread loads rows lr + 32 i of both tiles, 16 bytes at k chunk lc
+    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+    uint4 xr[4], wr[4];
+    int xrow[4], wrow[4];
+    float xw[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        xrow[i] = src_row[lr + 32 * i];
+        xw[i] = src_w[lr + 32 * i];
+        const int r = lr + 32 * i;                // row of the W tile -> row of the expert's matrix (-1: beyond the outputs)
+        const int n = GLU ? n0 + (r & 63) : n0 + r;
+        wrow[i] = n < N ? (GLU && r >= 64 ? N + n : n) : -1;
+    }
+    auto load = [&](int k0) {
+        const int k = k0 + lc * 8;
+        const bool kok = k < K;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint4 v = zero;
+            if (kok && xrow[i] >= 0) {
+                v = *reinterpret_cast<const uint4*>(X + (size_t)xrow[i] * ldx + k);
+                if (GLU) v = moe_scale8(v, xw[i]);
+            }
+            xr[i] = v;
+            uint4 u = zero;
+            if (kok && wrow[i] >= 0) u = *reinterpret_cast<const uint4*>(We + (size_t)wrow[i] * ldw + k);
+            wr[i] = u;
+        }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            *reinterpret_cast<uint4*>(&xs[(lr + 32 * i) * MOE_LD + lc * 8]) = xr[i];
+            *reinterpret_cast<uint4*>(&ws[(lr + 32 * i) * MOE_LD + lc * 8]) = wr[i];
+        }
+    };
+    f32x4 acc[4][4];
+#pragma unroll
+    for (int f = 0; f < 4; ++f)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) acc[f][g] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const int r16 = lane & 15, q = lane >> 4;
+    // fragment f of this wave in the W tile: GLU gate tiles 0, 1 and up tiles 2, 3 of outputs 32 wn ..; else outputs 64 wn ..
+    int wbase[4];
+#pragma unroll
+    for (int f = 0; f < 4; ++f) wbase[f] = GLU ? (f >> 1) * 64 + wn * 32 + (f & 1) * 16 : wn * 64 + f * 16;
+    const int my_rows = rows - wm * 64;           // rows of this wave's half that exist
+    const int groups = my_rows <= 0 ? 0 : (my_rows >= 64 ? 4 : (my_rows + 15) >> 4);
+    load(0);
+    for (int k0 = 0; k0 < K; k0 += MOE_KS) {
+        __syncthreads();           // the last step's readers are done
+        stage();
+        __syncthreads();
+        if (k0 + MOE_KS < K) load(k0 + MOE_KS);
+#pragma unroll
+        for (int ks = 0; ks < MOE_KS / 32; ++ks) {
+            uint4 a[4];
+#pragma unroll
+            for (int f = 0; f < 4; ++f) a[f] = *reinterpret_cast<const uint4*>(&ws[(wbase[f] + r16) * MOE_LD + ks * 32 + q * 8]);
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                if (g < groups) {
+                    const uint4 b = *reinterpret_cast<const uint4*>(&xs[(wm * 64 + g * 16 + r16) * MOE_LD + ks * 32 + q * 8]);
+#pragma unroll
+                    for (int f = 0; f < 4; ++f)
+                        acc[f][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[f]), __builtin_bit_cast(bf16x8, b),
+                                                                            acc[f][g], 0, 0, 0);
+                }
+            }
+        }
+    }
+    // lane holds rows m = 64 wm + 16 g + r16 and, of fragment f, the W rows 4 q + i
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const int m = wm * 64 + g * 16 + r16;
+        if (m >= rows) continue;
+        bf16* orow = out + (size_t)(place0 + m) * ld_out;
+#pragma unroll
+        for (int f = 0; f < (GLU ? 2 : 4); ++f) {
+            const int nb = GLU ? n0 + wn * 32 + f * 16 + q * 4 : n0 + wn * 64 + f * 16 + q * 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (nb + i < N) {
+                    float v = acc[f][g][i];
+                    if (GLU) v = moe_glu(v, acc[f + 2][g][i], limit, alpha);
+                    orow[nb + i] = from_f32<bf16>(v);
+                }
+            }
+        }
+    }
+}
+
 // Any dtype and size, FMA in ascending k.  Block 256 threads, tile 64 rows x 64 outputs, thread (ty, tx) owns rows
 // 4 ty .. 4 ty + 3 and outputs tx, tx + 16, tx + 32, tx + 48.
 template <typename T, bool GLU>
@@ -357,14 +487,22 @@ moe_gemm_plain_kernel(T* __restrict__ out, int ld_out, const T* __restrict__ X, 
 
 extern "C" int ilm_moe_gemm(void* out, int ld_out, const void* X, int ldx, const void* perm, int top, const void* pair_w, const void* W,
                             long w_expert, int ldw, const void* tiles, const void* n_tiles, int max_tiles, int N, int K, int glu,
-                            float limit, float alpha, int dtype, int force_plain, hipStream_t stream) {
+                            float limit, float alpha, int dtype, int force_plain, int tile_rows, hipStream_t stream) {
+    ILM_REQUIRE(tile_rows == MOE_TM || tile_rows == MOE_BM, "moe_gemm: tiles of %d rows (%d or %d)", tile_rows, MOE_TM, MOE_BM);
     ILM_REQUIRE(max_tiles > 0 && max_tiles <= 65535 && N > 0 && K > 0 && top > 0, "moe_gemm: bad sizes (tiles %d, N %d, K %d)", max_tiles, N, K);
     ILM_REQUIRE(ld_out >= N && ldx >= K && ldw >= K, "moe_gemm: rows shorter than their products");
     dim3 grid((N + MOE_TN - 1) / MOE_TN, max_tiles);
 #define MOE_ARGS(T__) (T__*)out, ld_out, (const T__*)X, ldx, (const int*)perm, top, (const float*)pair_w, (const T__*)W, (size_t)w_expert, ldw, \
                       (const int*)tiles, (const int*)n_tiles, N, K, limit, alpha
     const bool aligned = K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && w_expert % 8 == 0 && ((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0;
-    if (dtype == ILM_DTYPE_BF16 && aligned && !force_plain) {
+    if (dtype == ILM_DTYPE_BF16 && aligned && !force_plain && tile_rows == MOE_BM) {
+        dim3 big(max_tiles, glu ? (N + 63) / 64 : (N + 127) / 128);
+        ILM_REQUIRE(big.y <= 65535, "moe_gemm: %d outputs are too many", N);
+        if (glu) moe_gemm_mfma128_kernel<true><<<big, 256, 0, stream>>>(MOE_ARGS(bf16));
+        else moe_gemm_mfma128_kernel<false><<<big, 256, 0, stream>>>(MOE_ARGS(bf16));
+    } else if (tile_rows != MOE_TM) {
+        ILM_REQUIRE(false, "moe_gemm: tiles of %d rows are the bfloat16 matrix-core kernel's alone", tile_rows);
+    } else if (dtype == ILM_DTYPE_BF16 && aligned && !force_plain) {
         if (glu) moe_gemm_mfma_kernel<true><<<grid, 256, 0, stream>>>(MOE_ARGS(bf16));
         else moe_gemm_mfma_kernel<false><<<grid, 256, 0, stream>>>(MOE_ARGS(bf16));
     } else if (dtype == ILM_DTYPE_BF16) {

@@ -105,6 +105,99 @@ stream_update_kernel(void* __restrict__ x, float* __restrict__ r, const void* __
     for (int j = tid; j < H; j += SU_THREADS) st_any(x, (size_t)t * H + j, x_dt, row[j] * rstd_g[j / gs] * ld_any(w, j, w_dt));
 }
 
+
+// ---- the same with four elements a thread (rows, strides and pointers that allow 16-byte float and 8-byte bfloat16 accesses) ----
+__device__ __forceinline__ float4 ld4_any(const void* p, size_t i, int dt) {
+    if (dt == ILM_DTYPE_F32) return *reinterpret_cast<const float4*>((const float*)p + i);
+    const uint2 v = *reinterpret_cast<const uint2*>((const uint16_t*)p + i);
+    return make_float4(bf16_bits_to_f32((uint16_t)(v.x & 0xffffu)), bf16_bits_to_f32((uint16_t)(v.x >> 16)),
+                       bf16_bits_to_f32((uint16_t)(v.y & 0xffffu)), bf16_bits_to_f32((uint16_t)(v.y >> 16)));
+}
+__device__ __forceinline__ void st4_any(void* p, size_t i, int dt, float4 v) {
+    if (dt == ILM_DTYPE_F32) {
+        *reinterpret_cast<float4*>((float*)p + i) = v;
+    } else {
+        uint2 o;
+        o.x = (uint32_t)from_f32<bf16>(v.x).bits | ((uint32_t)from_f32<bf16>(v.y).bits << 16);
+        o.y = (uint32_t)from_f32<bf16>(v.z).bits | ((uint32_t)from_f32<bf16>(v.w).bits << 16);
+        *reinterpret_cast<uint2*>((uint16_t*)p + i) = o;
+    }
+}
+
+template <int THREADS>
+__global__ void __launch_bounds__(THREADS)
+stream_update_vec_kernel(void* __restrict__ x, float* __restrict__ r, const void* __restrict__ y, const void* __restrict__ z,
+                         const void* __restrict__ zb, const void* __restrict__ bw, const void* __restrict__ w, int H, int groups, int kind,
+                         float alpha, float eps_b, float eps, int x_dt, int y_dt, int z_dt, int w_dt, int parts, size_t part_stride,
+                         int y_stride, int z_stride) {
+    extern __shared__ float4 row4[];         // H floats
+    float* row = reinterpret_cast<float*>(row4);
+    __shared__ float red[THREADS / 64];
+    __shared__ float rstd_g[SU_MAX_GROUPS];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    float* rr = r + (size_t)t * H;
+    if (kind == SU_NONE) {
+        for (int j = tid * 4; j < H; j += THREADS * 4) *reinterpret_cast<float4*>(&row[j]) = *reinterpret_cast<const float4*>(&rr[j]);
+    } else {
+        float ss = 0.f;
+        for (int j = tid * 4; j < H; j += THREADS * 4) {
+            float4 v = ld4_any(y, (size_t)t * y_stride + j, y_dt);
+            for (int p = 1; p < parts; ++p) {
+                const float4 a = ld4_any(y, (size_t)p * part_stride + (size_t)t * y_stride + j, y_dt);
+                v.x += a.x, v.y += a.y, v.z += a.z, v.w += a.w;
+            }
+            *reinterpret_cast<float4*>(&row[j]) = v;
+            ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss))));
+        }
+        float f = alpha;
+        if (kind == SU_NORMED) f = alpha / sqrtf(block_sum<THREADS / 64>(ss, red) / (float)H + eps_b);
+        for (int j = tid * 4; j < H; j += THREADS * 4) {
+            float4 v = *reinterpret_cast<const float4*>(&row[j]);
+            v.x *= f, v.y *= f, v.z *= f, v.w *= f;
+            if (kind == SU_GATED) {
+                float4 g = ld4_any(z, (size_t)t * z_stride + j, z_dt);
+                if (zb != nullptr) {
+                    const float4 b = ld4_any(zb, j, w_dt);
+                    g.x += b.x, g.y += b.y, g.z += b.z, g.w += b.w;
+                }
+                v.x *= su_sigmoid(g.x), v.y *= su_sigmoid(g.y), v.z *= su_sigmoid(g.z), v.w *= su_sigmoid(g.w);
+            } else if (kind == SU_NORMED) {
+                const float4 b = ld4_any(bw, j, w_dt);
+                v.x *= b.x, v.y *= b.y, v.z *= b.z, v.w *= b.w;
+            }
+            float4 s = *reinterpret_cast<const float4*>(&rr[j]);
+            s.x += v.x, s.y += v.y, s.z += v.z, s.w += v.w;
+            *reinterpret_cast<float4*>(&rr[j]) = s;
+            *reinterpret_cast<float4*>(&row[j]) = s;
+        }
+    }
+    if (x == nullptr) return;
+    if (w == nullptr) {
+        for (int j = tid * 4; j < H; j += THREADS * 4) st4_any(x, (size_t)t * H + j, x_dt, *reinterpret_cast<const float4*>(&row[j]));
+        return;
+    }
+    __syncthreads();
+    const int gs = H / groups, wave = tid >> 6, lane = tid & 63;
+    for (int g = wave; g < groups; g += THREADS / 64) {
+        float ss = 0.f;
+        for (int j = lane; j < gs; j += 64) {
+            const float v = row[g * gs + j];
+            ss = fmaf(v, v, ss);
+        }
+        ss = wave_sum(ss);
+        if (lane == 0) rstd_g[g] = 1.0f / sqrtf(ss / (float)gs + eps);
+    }
+    __syncthreads();
+    for (int j = tid * 4; j < H; j += THREADS * 4) {
+        float4 v = *reinterpret_cast<const float4*>(&row[j]);
+        const float4 ww = ld4_any(w, j, w_dt);
+        v.x *= rstd_g[j / gs] * ww.x, v.y *= rstd_g[(j + 1) / gs] * ww.y, v.z *= rstd_g[(j + 2) / gs] * ww.z, v.w *= rstd_g[(j + 3) / gs] * ww.w;
+        st4_any(x, (size_t)t * H + j, x_dt, v);
+    }
+}
+
+static bool su_aligned(const void* p, int dt) { return p == nullptr || ((uintptr_t)p % (dt == ILM_DTYPE_F32 ? 16 : 8)) == 0; }
+
 extern "C" int ilm_stream_update(void* x, void* r, const void* y, const void* z, const void* zb, const void* bw, const void* w,
                                  int rows, int H, int groups, int kind, float alpha, float eps_b, float eps, int x_dt, int y_dt,
                                  int z_dt, int w_dt, int parts, long part_stride, int y_stride, int z_stride, hipStream_t stream) {
@@ -116,9 +209,18 @@ extern "C" int ilm_stream_update(void* x, void* r, const void* y, const void* z,
     ILM_REQUIRE(w == nullptr || (groups >= 1 && groups <= SU_MAX_GROUPS && H % groups == 0),
                 "stream_update: rows of %d do not divide into %d groups (at most %d)", H, groups, SU_MAX_GROUPS);
     ILM_REQUIRE(w == nullptr || x != nullptr, "stream_update: a norm needs an output");
-    stream_update_kernel<<<rows, SU_THREADS, (size_t)H * sizeof(float), stream>>>(
-        x, (float*)r, y, z, zb, bw, w, H, groups < 1 ? 1 : groups, kind, alpha, eps_b, eps, x_dt, y_dt, z_dt, w_dt, parts,
-        (size_t)part_stride, y_stride, z_stride);
+    const bool vec = H % 4 == 0 && y_stride % 4 == 0 && z_stride % 4 == 0 && part_stride % 4 == 0 && su_aligned(x, x_dt) && su_aligned(r, ILM_DTYPE_F32) &&
+                     su_aligned(y, y_dt) && su_aligned(z, z_dt) && su_aligned(zb, w_dt) && su_aligned(bw, w_dt) && su_aligned(w, w_dt);
+#define SU_ARGS x, (float*)r, y, z, zb, bw, w, H, groups < 1 ? 1 : groups, kind, alpha, eps_b, eps, x_dt, y_dt, z_dt, w_dt, parts, \
+                (size_t)part_stride, y_stride, z_stride
+    // (a row of up to 1,024 numbers gives 256 threads four each; wider rows of a launch that leaves compute units idle take 1,024 threads)
+    if (vec && H > 1024 && rows <= 2 * ilm_num_cus())
+        stream_update_vec_kernel<1024><<<rows, 1024, (size_t)H * sizeof(float), stream>>>(SU_ARGS);
+    else if (vec)
+        stream_update_vec_kernel<256><<<rows, 256, (size_t)H * sizeof(float), stream>>>(SU_ARGS);
+    else
+        stream_update_kernel<<<rows, SU_THREADS, (size_t)H * sizeof(float), stream>>>(SU_ARGS);
+#undef SU_ARGS
     ILM_LAUNCH_CHECK("stream_update");
     return 0;
 }

@@ -1595,17 +1595,20 @@ def softcap_(x: torch.Tensor, cap: float) -> torch.Tensor:
 
 # ---- many small experts of which a token uses a few -----------------------------------------------------------------------
 MOE_TILE_ROWS = 64       # rows of one expert a workgroup of the experts' products takes (ilm_moe_tile_rows())
+MOE_BIG_TILE_ROWS = 128  # the same for steps of many rows an expert (the bfloat16 matrix-core kernel with tiles of 128 x 128)
+MOE_BIG_MIN_ROWS = int(os.environ.get("INFINILM_AMD_MOE_BIG_MIN_ROWS", "96"))   # pairs an expert (on average) from which it runs
 MOE_FORCE_PLAIN = os.environ.get("INFINILM_AMD_MOE_PLAIN", "0") == "1"   # 1: the FMA products also in bfloat16
 
 
 class ExpertPlan:
     """Where every (token, slot) pair of a step lies once the pairs are ordered by expert."""
-    __slots__ = ("ids", "weights", "perm", "inv", "tiles", "n_tiles", "offsets", "max_tiles", "top", "pairs")
+    __slots__ = ("ids", "weights", "perm", "inv", "tiles", "n_tiles", "offsets", "max_tiles", "top", "pairs", "tile_rows")
 
 
-def moe_route(logits: torch.Tensor, experts: int, top: int) -> ExpertPlan:
+def moe_route(logits: torch.Tensor, experts: int, top: int, big_tiles_ok: bool = False) -> ExpertPlan:
     """From float32 router logits [T, >= experts] (the first `experts` entries of a row count): the `top` experts of every token
-    with sigmoid(logit) as their weights, and the pairs ordered by expert for `moe_gemm`."""
+    with sigmoid(logit) as their weights, and the pairs ordered by expert for `moe_gemm`.  `big_tiles_ok`: the products that
+    follow are bfloat16 with every K a multiple of 8, so a step of many pairs an expert may be cut into tiles of 128 rows."""
     _dev(logits)
     if logits.dtype != F32 or logits.dim() != 2 or logits.stride(1) != 1 or logits.shape[1] < experts:
         raise KernelError("router logits are float32 rows that hold every expert")
@@ -1617,7 +1620,8 @@ def moe_route(logits: torch.Tensor, experts: int, top: int) -> ExpertPlan:
     plan.ids = torch.empty((T, top), dtype=torch.int32, device=dev)
     plan.weights = torch.empty((T, top), dtype=F32, device=dev)
     _run("ilm_moe_route", plan.ids.data_ptr(), plan.weights.data_ptr(), logits.data_ptr(), T, int(experts), int(top), logits.stride(0), _stream())
-    plan.max_tiles = min(P, P // MOE_TILE_ROWS + min(experts, P))
+    plan.tile_rows = MOE_BIG_TILE_ROWS if big_tiles_ok and not MOE_FORCE_PLAIN and P >= MOE_BIG_MIN_ROWS * experts else MOE_TILE_ROWS
+    plan.max_tiles = min(P, P // plan.tile_rows + min(experts, P))
     book = torch.empty((experts + 1 + 2 * P + 3 * plan.max_tiles + 1,), dtype=torch.int32, device=dev)
     plan.offsets = book[:experts + 1]
     plan.perm = book[experts + 1:experts + 1 + P]
@@ -1625,7 +1629,7 @@ def moe_route(logits: torch.Tensor, experts: int, top: int) -> ExpertPlan:
     plan.tiles = book[experts + 1 + 2 * P:experts + 1 + 2 * P + 3 * plan.max_tiles]
     plan.n_tiles = book[-1:]
     _run("ilm_moe_sort", plan.offsets.data_ptr(), plan.perm.data_ptr(), plan.inv.data_ptr(), plan.tiles.data_ptr(), plan.n_tiles.data_ptr(),
-         plan.ids.data_ptr(), P, int(experts), plan.max_tiles, _stream())
+         plan.ids.data_ptr(), P, int(experts), plan.max_tiles, plan.tile_rows, _stream())
     return plan
 
 
@@ -1645,7 +1649,7 @@ def moe_gemm(x: torch.Tensor, w: torch.Tensor, plan: ExpertPlan, glu: bool, limi
     out = torch.empty((plan.pairs, N), dtype=x.dtype, device=x.device)
     _run("ilm_moe_gemm", out.data_ptr(), N, x.data_ptr(), x.stride(0), plan.perm.data_ptr(), plan.top, plan.weights.data_ptr() if glu else None,
          w.data_ptr(), Nw * K, K, plan.tiles.data_ptr(), plan.n_tiles.data_ptr(), plan.max_tiles, N, K, int(bool(glu)), float(limit),
-         float(alpha), _dt(x), int(MOE_FORCE_PLAIN), _stream(), label="ilm_moe_gemm (gate/up)" if glu else "ilm_moe_gemm (down)")
+         float(alpha), _dt(x), int(MOE_FORCE_PLAIN), plan.tile_rows, _stream(), label="ilm_moe_gemm (gate/up)" if glu else "ilm_moe_gemm (down)")
     return out
 
 

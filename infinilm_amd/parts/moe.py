@@ -69,7 +69,8 @@ class RoutedExperts(FeedForward):
 
     def forward(self, x, batch) -> torch.Tensor:
         logits = kernels.gemm(x, self.router.weight, None, 1.0, torch.float32)          # [T, experts (+ 1)]
-        plan = kernels.moe_route(logits, self.E, self.top)
+        plan = kernels.moe_route(logits, self.E, self.top,
+                                 big_tiles_ok=x.dtype == torch.bfloat16 and self.W % 8 == 0 and self.ff % 8 == 0 and x.stride(0) % 8 == 0)
         if RoutedExperts.trace is not None:
             RoutedExperts.trace.append(plan.ids.clone())
         act = kernels.moe_gemm(x, self.w_gate_up, plan, True, self.limit, self.alpha)   # [pairs, ff], ordered by expert

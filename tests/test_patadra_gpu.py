@@ -147,7 +147,7 @@ def _experts(dtype, W, E, top, ff, limit, shared_ff, shared_limit, width):
 
 @pytest.mark.parametrize("dtype", [F32, BF])
 @pytest.mark.parametrize("T,width,E,top,ff,shared_ff", [(1, 64, 4, 2, 48, 40), (5, 96, 3, 1, 40, 0), (200, 64, 3, 2, 100, 24), (70, 100, 8, 3, 36, 20),
-                                                        (300, 128, 2, 2, 64, 0), (33, 72, 16, 1, 8, 8), (150, 256, 8, 2, 192, 64)])
+                                                        (300, 128, 2, 2, 64, 0), (33, 72, 16, 1, 8, 8), (150, 256, 8, 2, 192, 64), (700, 256, 4, 2, 136, 0), (1000, 192, 3, 3, 200, 64)])
 def test_routed_experts_against_the_formula(T, width, E, top, ff, shared_ff, dtype):
     """The feed-forward alone: one token, few, and so many that an expert's rows fill several tiles; widths and inner sizes
     that are no multiples of 8 or 64 (the plain products in bfloat16 too); the score at the expert's input, limits that bind."""
