@@ -66,7 +66,7 @@ _SIGNATURES = {
     "ilm_softcap": [_P, _L, _F, _P],
     "ilm_moe_route": [_P, _P, _P, _I, _I, _I, _I, _P],
     "ilm_moe_sort": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
-    "ilm_moe_gemm": [_P, _I, _P, _I, _P, _I, _P, _P, _L, _I, _P, _P, _I, _I, _I, _I, _F, _F, _I, _I, _I, _P],
+    "ilm_moe_gemm": [_P, _I, _P, _I, _P, _I, _P, _P, _L, _I, _P, _P, _I, _I, _I, _I, _F, _F, _I, _I, _I, _I, _P],
     "ilm_moe_combine": [_P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _P],
     "ilm_glu_clamp": [_P, _P, _I, _I, _I, _F, _F, _I, _P],
     "ilm_head_gemm": [_P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _L, _I, _I, _P],

@@ -133,6 +133,23 @@ def test_routing_takes_the_largest_scores(E, top):
     assert int(offs[E]) == T * top
 
 
+def test_routing_of_rows_without_numbers_stays_in_range():
+    """A row of NaNs compares larger nowhere: it still gets valid experts, and every pair keeps its place in the order."""
+    from infinilm_amd import kernels
+    E, top, T = 6, 2, 9
+    z = torch.randn(T, E, generator=torch.Generator().manual_seed(3))
+    z[2] = float("nan")
+    z[5, 1:] = float("nan")
+    z[7] = float("-inf")
+    plan = kernels.moe_route(z.to(DEV), E, top)
+    ids = plan.ids.cpu().long()
+    assert int(ids.min()) >= 0 and int(ids.max()) < E
+    perm, inv = plan.perm.cpu().long(), plan.inv.cpu().long()
+    assert sorted(perm.tolist()) == list(range(T * top)) and torch.equal(perm[inv], torch.arange(T * top))
+    assert int(plan.offsets.cpu()[E]) == T * top
+    assert ids[5, 0] == 0
+
+
 def _experts(dtype, W, E, top, ff, limit, shared_ff, shared_limit, width):
     from infinilm_amd.config.spec import PartSpec
     from infinilm_amd.parts import BuildContext
@@ -181,6 +198,15 @@ def test_routed_experts_against_the_formula(T, width, E, top, ff, shared_ff, dty
         _close(got.cpu(), want, 1e-5, "float32 experts")
     g_all = torch.einsum("tk,enk->ten", h.double(), torch.stack([Wd[f"l0.mlp.e{e}.gate"] for e in range(E)]))
     assert float(g_all.max()) > 0.8, "no gate reaches the limit: it would show nothing"
+
+
+@pytest.mark.parametrize("T,width,E,top,ff,shared_ff", [(700, 256, 4, 2, 136, 0), (900, 320, 3, 2, 264, 0), (1000, 192, 3, 3, 200, 64)])
+def test_routed_experts_in_wide_tiles(T, width, E, top, ff, shared_ff, monkeypatch):
+    """The many-rows kernel with 256 rows of W a tile (an option): output slices that end inside a tile, experts with more and
+    fewer rows than a tile."""
+    from infinilm_amd import kernels
+    monkeypatch.setattr(kernels, "MOE_WIDE", 1)
+    test_routed_experts_against_the_formula(T, width, E, top, ff, shared_ff, BF)
 
 
 # ---- the attention alone, with one key made to stand out ----------------------------------------------------------------
