@@ -136,6 +136,84 @@ head_gemm_kernel(TO* __restrict__ out, const T* __restrict__ x, const T* __restr
         }
 }
 
+// The same for few rows of bfloat16 on the matrix cores: a wave owns one head and 16 outputs for up to 64 rows (four row tiles
+// that share every fragment of W), k in steps of 32 with all of a step's loads independent of each other; nothing passes LDS.
+// x rows, K and the strides of x in multiples of 8 elements (16-byte loads); W with k dense (16-byte loads) or n dense (eight
+// 2-byte loads a fragment).  A row's sum is its own: rows beyond T are zeros and are not stored.
+typedef __attribute__((ext_vector_type(8))) __bf16 hg_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float hg_f32x4;
+
+template <bool W_K_DENSE>
+__global__ void __launch_bounds__(256)
+head_gemm_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ x, const bf16* __restrict__ w, int M, int N, int K, int H,
+                      long x_t, long x_h, long w_h, long w_k, long w_n, long o_t, long o_h) {
+    const int n_tiles = (N + 15) >> 4;
+    const int item = blockIdx.x * 4 + (threadIdx.x >> 6);          // (head, tile of 16 outputs)
+    if (item >= H * n_tiles) return;
+    const int h = item / n_tiles, n0 = (item % n_tiles) * 16, m0 = blockIdx.y * 64;
+    const int lane = threadIdx.x & 63, r16 = lane & 15, q = lane >> 4;
+    const bf16* xh = x + (size_t)h * x_h;
+    const bf16* wh = w + (size_t)h * w_h;
+    const int n = n0 + r16;
+    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+    hg_f32x4 acc[4];
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt) acc[rt] = hg_f32x4{0.f, 0.f, 0.f, 0.f};
+    const int row_tiles = (M - m0 + 15) >> 4 < 4 ? (M - m0 + 15) >> 4 : 4;
+#pragma unroll 2
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        const int k = k0 + q * 8;
+        uint4 b = zero;
+        if (k < K && n < N) {
+            if (W_K_DENSE) {
+                b = *reinterpret_cast<const uint4*>(wh + (size_t)n * w_n + k);
+            } else {
+                uint32_t e[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) e[j] = (wh + (size_t)(k + j) * w_k)[n].bits;
+                b = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16));
+            }
+        }
+        uint4 a[4];
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) {
+            const int m = m0 + rt * 16 + r16;
+            a[rt] = (rt < row_tiles && m < M && k < K) ? *reinterpret_cast<const uint4*>(xh + (size_t)m * x_t + k) : zero;
+        }
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt)
+            if (rt < row_tiles)
+                acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(hg_bf16x8, a[rt]), __builtin_bit_cast(hg_bf16x8, b),
+                                                                  acc[rt], 0, 0, 0);
+    }
+    // lane holds rows m0 + 16 rt + 4 q + i and output n
+    if (n < N)
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int m = m0 + rt * 16 + q * 4 + i;
+                if (rt < row_tiles && m < M) out[(size_t)m * o_t + (size_t)h * o_h + n] = from_f32<bf16>(acc[rt][i]);
+            }
+}
+
+extern "C" int ilm_head_gemm_mfma(void* out, const void* x, const void* w, int M, int N, int K, int H, long x_t, long x_h, long w_h,
+                                  long w_k, long w_n, long o_t, long o_h, hipStream_t stream) {
+    ILM_REQUIRE(M > 0 && N > 0 && K > 0 && H > 0, "head_gemm_mfma: bad sizes");
+    ILM_REQUIRE(K % 8 == 0 && x_t % 8 == 0 && x_h % 8 == 0 && ((uintptr_t)x % 16) == 0, "head_gemm_mfma: rows of x must allow 16-byte loads");
+    ILM_REQUIRE(w_k == 1 || w_n == 1, "head_gemm_mfma: one axis of W must be dense");
+    ILM_REQUIRE(w_k != 1 || (w_n % 8 == 0 && w_h % 8 == 0 && ((uintptr_t)w % 16) == 0), "head_gemm_mfma: rows of W must allow 16-byte loads");
+    const long items = (long)H * ((N + 15) / 16);
+    ILM_REQUIRE(items < (1L << 30) && (M + 63) / 64 <= 65535, "head_gemm_mfma: too large");
+    dim3 grid((unsigned)((items + 3) / 4), (M + 63) / 64);
+    if (w_k == 1)
+        head_gemm_mfma_kernel<true><<<grid, 256, 0, stream>>>((bf16*)out, (const bf16*)x, (const bf16*)w, M, N, K, H, x_t, x_h, w_h, w_k, w_n, o_t, o_h);
+    else
+        head_gemm_mfma_kernel<false><<<grid, 256, 0, stream>>>((bf16*)out, (const bf16*)x, (const bf16*)w, M, N, K, H, x_t, x_h, w_h, w_k, w_n, o_t, o_h);
+    ILM_LAUNCH_CHECK("head_gemm_mfma");
+    return 0;
+}
+
 extern "C" int ilm_head_gemm(void* out, const void* x, const void* w, int M, int N, int K, int H, long x_t, long x_h, long w_h,
                              long w_k, long w_n, long o_t, long o_h, int dtype, int out_dt, hipStream_t stream) {
     ILM_REQUIRE(M > 0 && N > 0 && K > 0 && H > 0 && H <= 65535, "head_gemm: bad sizes");

@@ -70,6 +70,7 @@ _SIGNATURES = {
     "ilm_moe_combine": [_P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _P],
     "ilm_glu_clamp": [_P, _P, _I, _I, _I, _F, _F, _I, _P],
     "ilm_head_gemm": [_P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _L, _I, _I, _P],
+    "ilm_head_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _L, _P],
     "ilm_group_norm_gate": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _I, _I, _L, _P],
     "ilm_causal_conv": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P],
     "ilm_ssm_steps": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P],

@@ -1477,6 +1477,7 @@ def latent_prep(rows: torch.Tensor, qx: torch.Tensor, positions: torch.Tensor, f
 
 
 HEAD_GEMM_LIBRARY_MIN_ROWS = 33   # rows from which the bfloat16 product per head goes to the vendor library
+HEAD_GEMM_MFMA_MAX_ROWS = int(os.environ.get("INFINILM_AMD_HEAD_GEMM_MFMA_MAX_ROWS", "128"))   # rows up to which it takes the matrix-core kernel without LDS (0: never)
 
 
 def head_gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
@@ -1488,6 +1489,13 @@ def head_gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tens
     if tuple(w.shape) != (H, K, N) or tuple(out.shape) != (T, H, N) or x.stride(2) != 1 or out.stride(2) != 1 \
             or x.dtype != w.dtype or (w.stride(1) != 1 and w.stride(2) != 1):
         raise KernelError(f"a product per head of {tuple(x.shape)} x {tuple(w.shape)} -> {tuple(out.shape)} does not fit")
+    if (x.dtype == BF16 and out.dtype == BF16 and T <= HEAD_GEMM_MFMA_MAX_ROWS and not FORCE_BASIC and K % 8 == 0
+            and x.stride(0) % 8 == 0 and x.stride(1) % 8 == 0 and x.data_ptr() % 16 == 0
+            and (w.stride(1) != 1 or (w.stride(2) % 8 == 0 and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0))):
+        # few rows (decoded tokens): a wave a head and 16 outputs on the matrix cores, nothing through LDS
+        _run("ilm_head_gemm_mfma", out.data_ptr(), x.data_ptr(), w.data_ptr(), T, N, K, H, x.stride(0), x.stride(1), w.stride(0),
+             w.stride(1), w.stride(2), out.stride(0), out.stride(1), _stream())
+        return out
     if x.dtype == BF16 and out.dtype == BF16 and T >= HEAD_GEMM_LIBRARY_MIN_ROWS and USE_LIBRARY_GEMM and not FORCE_BASIC:
         with _timed("library_gemm"):
             out.copy_(torch.bmm(x.transpose(0, 1), w).transpose(0, 1))

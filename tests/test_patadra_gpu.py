@@ -133,6 +133,37 @@ def test_routing_takes_the_largest_scores(E, top):
     assert int(offs[E]) == T * top
 
 
+@pytest.mark.parametrize("T,H,K,N", [(1, 2, 8, 20), (5, 3, 16, 40), (40, 4, 64, 96), (64, 6, 32, 48), (100, 2, 136, 24), (128, 8, 128, 128),
+                                     (7, 32, 128, 64), (17, 5, 72, 17)])
+def test_product_per_head_for_few_rows_on_the_matrix_cores(T, H, K, N):
+    """Rows whose strides allow 16-byte loads take the kernel without LDS: both layouts of W, outputs that end inside a tile of
+    16, K that ends inside a step of 32, more rows than one workgroup's 64, columns beside the result left alone, and a row's
+    result the same bits whatever rows lie beside it."""
+    from infinilm_amd import kernels
+    assert T <= kernels.HEAD_GEMM_MFMA_MAX_ROWS
+    g = torch.Generator().manual_seed(T + K)
+    x = torch.randn(T, H * (K + 8), generator=g).to(BF)
+    w_kn = (torch.randn(H, K, N, generator=g) / K ** 0.5).to(BF)
+    w_nk = (torch.randn(H, N, K, generator=g) / K ** 0.5).to(BF)
+    xv = x.to(DEV).view(T, H, K + 8)[:, :, :K]
+    kernels.enable_timing(True)
+    try:
+        kernels.timing_report()
+        out = torch.zeros(T, H, N + 3, dtype=BF, device=DEV)
+        kernels.head_gemm(xv, w_kn.to(DEV), out[:, :, :N])
+        out2 = torch.empty(T, H, N, dtype=BF, device=DEV)
+        kernels.head_gemm(xv, w_nk.to(DEV).transpose(1, 2), out2)
+        assert set(kernels.timing_report()) == {"ilm_head_gemm_mfma"}, "the matrix-core kernel did not run"
+    finally:
+        kernels.enable_timing(False)
+    _close(out[:, :, :N].cpu(), torch.einsum("thk,hkn->thn", xv.cpu().double(), w_kn.double()), 1e-2, "W with the outputs dense")
+    assert float(out[:, :, N:].abs().max()) == 0.0
+    _close(out2.cpu(), torch.einsum("thk,hnk->thn", xv.cpu().double(), w_nk.double()), 1e-2, "W with the inputs dense")
+    one = torch.empty(1, H, N, dtype=BF, device=DEV)
+    kernels.head_gemm(xv[T - 1:], w_nk.to(DEV).transpose(1, 2), one)
+    assert torch.equal(one[0], out2[T - 1])
+
+
 def test_routing_of_rows_without_numbers_stays_in_range():
     """A row of NaNs compares larger nowhere: it still gets valid experts, and every pair keeps its place in the order."""
     from infinilm_amd import kernels
