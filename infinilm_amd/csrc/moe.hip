@@ -280,7 +280,8 @@ moe_gemm_mfma_kernel(bf16* __restrict__ out, int ld_out, const bf16* __restrict_
 // gate and up of 32 outputs, so the activation has both in one thread): 16 products for 8 fragment reads a k-step.  WN = 4
 // reads a third fewer bytes a product from the caches than WN = 2 (a tile's operands: 128 + 256 rows for 128 x 256 results).
 template <bool GLU, int WN>
-__global__ void __launch_bounds__(128 * WN)
+// (Three waves a SIMD: left to itself the compiler takes 170 registers a lane, two more than three workgroups a compute unit allow.)
+__global__ void __launch_bounds__(128 * WN) __attribute__((amdgpu_waves_per_eu(3, 3)))
 moe_gemm_mfma128_kernel(bf16* __restrict__ out, int ld_out, const bf16* __restrict__ X, int ldx, const int* __restrict__ perm, int top,
                         const float* __restrict__ pair_w, const bf16* __restrict__ W, size_t w_expert, int ldw, const int* __restrict__ tiles,
                         const int* __restrict__ n_tiles, int N, int K, float limit, float alpha, int n_slices) {
