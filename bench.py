@@ -51,7 +51,7 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 32 / 64 points, the prefill and the 32-bit record")
     ap.add_argument("--no-fp32", action="store_true", help="skip the 32-bit record (bfloat16 runs only)")
     ap.add_argument("--designs", action="store_true",
-                    help="instead of the default workload: prefill and decode throughput of the Kekevik design beside MiniCPM4 "
+                    help="instead of the default workload: prefill and decode throughput of another design (--design) beside MiniCPM4 "
                          "at equal layer sizes (random weights), with the time and the roofline share of every kernel")
     ap.add_argument("--design-shapes", default="1024,4096", help="widths to compare with --designs")
     ap.add_argument("--design", default="kekevik", choices=["kekevik", "pugavik", "patadra"],
