@@ -40,6 +40,7 @@ class _Group:
     window: int
     entries: List[int]
     pool: PagePool
+    keep_first: int = 0          # with a window: the sequence's first positions whose pages are never given back
 
 
 @dataclass
@@ -73,6 +74,15 @@ class StateView:
         self.pool, self.state_in, self.state_out = pool, state_in, state_out
 
 
+class Lent:
+    """What a block's forward gets when its run reads a second cache entry beside its own: `own` is the view of the
+    run's own entry (None: it has none), `lent` the read-only view of the entry it borrows."""
+    __slots__ = ("own", "lent")
+
+    def __init__(self, own, lent):
+        self.own, self.lent = own, lent
+
+
 class CacheManager:
     def __init__(self, needs: Sequence, page_size: int, num_pages: int, max_requests: int,
                  dtype: torch.dtype, device, num_pages_per_group: Optional[Dict[int, int]] = None,
@@ -99,11 +109,12 @@ class CacheManager:
         by_window: Dict[int, int] = {}
         for e, need in self._members:
             if isinstance(need, PagedKV):
-                if need.window not in by_window:
+                kept = need.keep_first if need.window > 0 else 0
+                if (need.window, kept) not in by_window:
                     n = (num_pages_per_group or {}).get(need.window, num_pages)
-                    by_window[need.window] = len(self.groups)
-                    self.groups.append(_Group(need.window, [], PagePool(n)))
-                g = by_window[need.window]
+                    by_window[(need.window, kept)] = len(self.groups)
+                    self.groups.append(_Group(need.window, [], PagePool(n), kept))
+                g = by_window[(need.window, kept)]
                 self.groups[g].entries.append(e)
                 self.group_of_entry[e] = g
         # data plane
@@ -163,7 +174,7 @@ class CacheManager:
 
     def stats(self) -> dict:
         return {"requests": len(self.requests),
-                "groups": [{"window": g.window, "entries": len(g.entries), "pages": g.pool.num_pages,
+                "groups": [{"window": g.window, "keep_first": g.keep_first, "entries": len(g.entries), "pages": g.pool.num_pages,
                             "free": g.pool.num_free, "idle": g.pool.num_idle, "evictions": g.pool.evictions,
                             "high_water": g.pool.high_water} for g in self.groups],
                 "state_slots_free": len(self._free_slots),
@@ -280,7 +291,7 @@ class CacheManager:
                 self._publish(r, tokens)
         for g, table in zip(self.groups, r.tables):
             first = self._first_needed_page(g, r.length)  # the next query sits at position `length`
-            for i in range(min(first, len(table))):
+            for i in range(-(-g.keep_first // self.page_size), min(first, len(table))):   # (the pages of the kept first positions stay)
                 if table[i] >= 0:
                     g.pool.give_back([table[i]])
                     table[i] = -1

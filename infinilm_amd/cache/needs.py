@@ -11,10 +11,12 @@ import torch
 @dataclass(frozen=True)
 class PagedKV:
     """Keys and values of every token, in pages.  window > 0: only the last `window` positions
-    before (and including) a query are ever read, so older pages can be given back."""
+    before (and including) a query are ever read, so older pages can be given back; keep_first > 0:
+    the sequence's first `keep_first` positions are read as well, so the pages that hold them stay."""
     num_kv_heads: int
     head_dim: int
     window: int = 0
+    keep_first: int = 0
 
 
 @dataclass(frozen=True)

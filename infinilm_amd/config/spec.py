@@ -41,11 +41,15 @@ class LayerRun:
     """One entry of the execution order: run `layer` with cache entry `cache`.
 
     A layer may appear in several runs (its weights are shared).  Two runs may name the same cache
-    entry: the one with `writes_cache` fills it, the others only read it."""
+    entry: the one with `writes_cache` fills it, the others only read it.  `borrows`: a second cache
+    entry, written by an earlier run, that this run reads beside its own (a layer that attends over
+    another layer's keys and values and keeps a state of its own): the block's view is then
+    `Lent(own, lent)`."""
     layer: int
     cache: Optional[int]
     writes_cache: bool = True
     start: Optional[RunStart] = None
+    borrows: Optional[int] = None
 
 
 @dataclass
@@ -87,7 +91,7 @@ class ModelSpec:
     shared_tensors: Optional[Dict[str, tuple]] = None
 
     def num_cache_entries(self) -> int:
-        ids = [r.cache for r in self.order if r.cache is not None]
+        ids = [r.cache for r in self.order if r.cache is not None] + [r.borrows for r in self.order if r.borrows is not None]
         return (max(ids) + 1) if ids else 0
 
     def validate(self) -> None:
@@ -109,3 +113,5 @@ class ModelSpec:
             if run.cache is not None and not run.writes_cache:
                 if run.cache not in writers or writers[run.cache] > i:
                     raise ValueError(f"order[{i}] reads cache entry {run.cache} before any run has written it")
+            if run.borrows is not None and (run.borrows not in writers or writers[run.borrows] >= i):
+                raise ValueError(f"order[{i}] borrows cache entry {run.borrows}, which no earlier run writes")

@@ -6,7 +6,7 @@
 //       (2i, 2i + 1), i < rd / 2, by the angle pos * freq[i], every value head divided by its root mean square
 //       over its first dv entries (or not); q and k are rewritten in place, k and v go to the paged cache.
 //   ilm_attn_headmix            raw_g(j) = scale q_g . k_kv(g),j;  s_h(j) = sum_g M[h, g] raw_g(j);  over the keys j
-//       the token sees (its last `window` positions, or all): p_h(j) = exp(s_h(j)) / (sum_j' exp(s_h(j')) + exp(sink_h));
+//       the token sees (its last `window` positions and the sequence's first `keep_first`, or all): p_h(j) = exp(s_h(j)) / (sum_j' exp(s_h(j')) + exp(sink_h));
 //       o_h = sum_j p_h(j) v_kv(h),j.  M and sink may be absent (identity, no term).
 //
 // All arithmetic is float.  The attention is the plain form: one block a token walks the keys in tiles of 64 aligned
@@ -119,7 +119,7 @@ attn_headmix_kernel(T* __restrict__ out, const T* __restrict__ q, const T* __res
                     const int* __restrict__ block_tables, const int* __restrict__ seg, const int* __restrict__ pos,
                     const int* __restrict__ rows, const float* __restrict__ mix, const float* __restrict__ sink,
                     int nh, int nkv, int d, int dv, int page, int max_blocks, int q_stride, int out_stride, float scale,
-                    int window) {
+                    int window, int keep_first) {
     extern __shared__ float smem[];
     float* qs = smem;
     float* raw = qs + nh * d;
@@ -134,6 +134,7 @@ attn_headmix_kernel(T* __restrict__ out, const T* __restrict__ q, const T* __res
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int p = pos[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int keep = lo < keep_first ? lo : keep_first;     // the first tokens stay seen below the window's edge: keys 0 .. keep - 1
     const int* bt = block_tables + (size_t)seg[t] * max_blocks;
     const T* qrow = q + (size_t)t * q_stride;
     const int per = nh / nkv;
@@ -143,9 +144,10 @@ attn_headmix_kernel(T* __restrict__ out, const T* __restrict__ q, const T* __res
     for (int i = tid; i < nh * dv; i += 256) acc[i] = 0.f;
     __syncthreads();
     const int chunks = (per + HM_R - 1) / HM_R;      // pieces of a group of at most HM_R heads
-    for (int tile = lo >> 6; tile <= (p >> 6); ++tile) {
+    for (int tile = keep > 0 ? 0 : lo >> 6; tile <= (p >> 6); ++tile) {
+        if ((tile << 6) + 63 < lo && (tile << 6) >= keep) continue;       // between the kept keys and the window
         const int key = (tile << 6) + lane;
-        const bool valid = key >= lo && key <= p;
+        const bool valid = key <= p && (key >= lo || key < keep);
         // 1. raw scores of all heads for the tile's keys: a wave takes (group, piece) items in turn, a lane a key
         for (int item = wave; item < nkv * chunks; item += 4) {
             const int c = item / chunks, g0 = c * per + (item % chunks) * HM_R;
@@ -197,32 +199,35 @@ attn_headmix_kernel(T* __restrict__ out, const T* __restrict__ q, const T* __res
             if (lane == 0) { run_m[h] = m_new; run_l[h] = l_new; corr[h] = cf; }
         }
         __syncthreads();
-        // 3. outputs: a thread takes (head, value entry) items in turn and walks the tile's keys in ascending order
-        const int j0 = lo > (tile << 6) ? lo - (tile << 6) : 0;
-        const int j1 = (p - (tile << 6)) < 63 ? p - (tile << 6) : 63;
+        // 3. outputs: a thread takes (head, value entry) items in turn and walks the tile's seen keys in ascending order: the
+        //    kept first keys, then the window's
         for (int idx = tid; idx < nh * dv; idx += 256) {
             const int h = idx / dv, e = idx % dv, c = h / per;
             float a = acc[idx] * corr[h];
             const float* wrow = wt + h * 64;
-            int j = j0;
-            if (VEC) {
-                for (; j <= j1 && (j & 3); ++j) {
+            for (int part = keep > (tile << 6) ? 0 : 1; part < 2; ++part) {
+                const int j0 = part == 0 ? 0 : (lo > (tile << 6) ? lo - (tile << 6) : 0);
+                const int j1 = part == 0 ? min(63, keep - 1 - (tile << 6)) : ((p - (tile << 6)) < 63 ? p - (tile << 6) : 63);
+                int j = j0;
+                if (VEC) {
+                    for (; j <= j1 && (j & 3); ++j) {
+                        const int kk = (tile << 6) + j;
+                        a = fmaf(wrow[j], to_f32(vc[(((size_t)bt[kk / page] * nkv + c) * d + e) * page + (kk % page)]), a);
+                    }
+                    for (; j + 3 <= j1; j += 4) {
+                        const int kk = (tile << 6) + j;
+                        float vv[4];
+                        hm_load4(vc + (((size_t)bt[kk / page] * nkv + c) * d + e) * page + (kk % page), vv);
+                        a = fmaf(wrow[j], vv[0], a);
+                        a = fmaf(wrow[j + 1], vv[1], a);
+                        a = fmaf(wrow[j + 2], vv[2], a);
+                        a = fmaf(wrow[j + 3], vv[3], a);
+                    }
+                }
+                for (; j <= j1; ++j) {
                     const int kk = (tile << 6) + j;
                     a = fmaf(wrow[j], to_f32(vc[(((size_t)bt[kk / page] * nkv + c) * d + e) * page + (kk % page)]), a);
                 }
-                for (; j + 3 <= j1; j += 4) {
-                    const int kk = (tile << 6) + j;
-                    float vv[4];
-                    hm_load4(vc + (((size_t)bt[kk / page] * nkv + c) * d + e) * page + (kk % page), vv);
-                    a = fmaf(wrow[j], vv[0], a);
-                    a = fmaf(wrow[j + 1], vv[1], a);
-                    a = fmaf(wrow[j + 2], vv[2], a);
-                    a = fmaf(wrow[j + 3], vv[3], a);
-                }
-            }
-            for (; j <= j1; ++j) {
-                const int kk = (tile << 6) + j;
-                a = fmaf(wrow[j], to_f32(vc[(((size_t)bt[kk / page] * nkv + c) * d + e) * page + (kk % page)]), a);
             }
             acc[idx] = a;
         }
@@ -249,7 +254,8 @@ extern "C" long ilm_attn_headmix_lds_bytes(int nh, int d, int dv) {
 extern "C" int ilm_attn_headmix(void* out, const void* q, const void* kc, const void* vc, const void* block_tables,
                                 const void* seg, const void* pos, const void* rows, int n_rows, const void* mix,
                                 const void* sink, int nh, int nkv, int d, int dv, int page, int max_blocks, int q_stride,
-                                int out_stride, float scale, int window, int dtype, hipStream_t stream) {
+                                int out_stride, float scale, int window, int keep_first, int dtype, hipStream_t stream) {
+    ILM_REQUIRE(keep_first >= 0, "attn_headmix: %d kept first tokens", keep_first);
     ILM_REQUIRE(n_rows > 0 && nh > 0 && nkv > 0 && d > 0 && page > 0 && max_blocks > 0, "attn_headmix: bad sizes");
     ILM_REQUIRE(nh % nkv == 0, "attn_headmix: %d query heads do not divide into %d groups", nh, nkv);
     ILM_REQUIRE(dv > 0 && dv <= d, "attn_headmix: value size %d in heads of %d", dv, d);
@@ -267,7 +273,7 @@ extern "C" int ilm_attn_headmix(void* out, const void* q, const void* kc, const 
         kern<<<n_rows, 256, shm, stream>>>((T_*)out, (const T_*)q, (const T_*)kc, (const T_*)vc, (const int*)block_tables, \
                                            (const int*)seg, (const int*)pos, (const int*)rows, (const float*)mix,        \
                                            (const float*)sink, nh, nkv, d, dv, page, max_blocks, q_stride, out_stride,   \
-                                           scale, window);                                                               \
+                                           scale, window, keep_first);                                                   \
     }
     if (dtype == ILM_DTYPE_F32) {
         if (vec) HM_LAUNCH(float, true) else HM_LAUNCH(float, false)

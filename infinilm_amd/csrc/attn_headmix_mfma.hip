@@ -5,7 +5,7 @@
 // so head h asks with a query of C d entries against the key row [k_0,j | ... | k_{C-1},j] of all groups, and takes its
 // values from its own group.  `ilm_headmix_queries` forms q' (float sums, bfloat16 result: a query like any other
 // operand of the score product); `ilm_attn_headmix_mfma` is then a flash attention over the window with one more term
-// exp(sink_h) in the denominator.  Cost of the score product: C times that of unmixed heads, and no exchange of scores
+// exp(sink_h) in the denominator (and, with `keep_first`, over the sequence's first keys as well).  Cost of the score product: C times that of unmixed heads, and no exchange of scores
 // between heads; for many groups the plain kernel's explicit mixing does less work.
 //
 // A workgroup = one item (a tile of up to 16 consecutive tokens of a request, or a single token) x one pass of 4 HPW
@@ -103,7 +103,7 @@ attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, co
                          const int* __restrict__ block_tables, const int* __restrict__ seg, const int* __restrict__ pos,
                          const int* __restrict__ tiles, int n_tiles, const int* __restrict__ singles,
                          const float* __restrict__ sink, int nh, int page, int max_blocks, int out_stride, float scale_log2e,
-                         int window, float* __restrict__ ws, int chunk_keys, const int* __restrict__ seg_offsets) {
+                         int window, float* __restrict__ ws, int chunk_keys, const int* __restrict__ seg_offsets, int keep_first) {
     constexpr int D = D32 * 32, KROW = D + 8, VROW = TK + 8, NS = TK / 16, NP = TK / 32;
     extern __shared__ __attribute__((aligned(16))) unsigned char hx_smem[];
     bf16* Ks = reinterpret_cast<bf16*>(hx_smem);                 // [NC][32][KROW]
@@ -190,8 +190,18 @@ attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, co
             if (pc < VPIECES && pg >= 0) vreg[i] = *reinterpret_cast<const uint4*>(vc + (((size_t)pg * NC + c) * D + row) * page + off + piece * 8);
         }
     };
-    if (kb_begin <= kb_end) fetch(kb_begin);
-    for (int kb = kb_begin; kb <= kb_end; kb += TK) {
+    // The first `keep_first` keys of the sequence stay seen below the window's edge: their tiles go first (in the chunked form:
+    // in chunk 0), then the tiles from the window's edge on.  Tile i of the walk begins at key tile_key(i).
+    int n_pre = 0;
+    if (keep_first > 0 && (chunk_keys == 0 || blockIdx.z == 0)) {
+        const int edge = lo_first & ~(TK - 1);                   // (the window's tiles begin here; kept keys from here on are theirs)
+        n_pre = (min(keep_first, edge) + TK - 1) / TK;
+    }
+    const int n_main = kb_begin <= kb_end ? (kb_end - kb_begin) / TK + 1 : 0;
+    auto tile_key = [&](int i) { return i < n_pre ? i * TK : kb_begin + (i - n_pre) * TK; };
+    if (n_pre + n_main > 0) fetch(tile_key(0));
+    for (int ti = 0; ti < n_pre + n_main; ++ti) {
+        const int kb = tile_key(ti);
         __syncthreads();                                         // the tile before this one has been read by every wave
 #pragma unroll
         for (int i = 0; i < KPER; ++i) {
@@ -206,7 +216,7 @@ attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, co
             if (pc < VPIECES) *reinterpret_cast<uint4*>(Vs + (c * D + row) * VROW + piece * 8) = vreg[i];
         }
         __syncthreads();
-        if (kb + TK <= kb_end) fetch(kb + TK);
+        if (ti + 1 < n_pre + n_main) fetch(tile_key(ti + 1));
         // head by head (a version that read every key and value fragment from LDS once for all heads of a wave kept more
         // registers live and measured slower: 455 against 374 us a prompt step at 32 heads of 128)
 #pragma unroll
@@ -232,7 +242,7 @@ attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, co
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int key = kb + s * 16 + g4 * 4 + j;
-                    const bool seen = tok_ok && key >= lo_tok && key <= p_tok;
+                    const bool seen = tok_ok && key <= p_tok && (key >= lo_tok || key < keep_first);
                     sc[s * 4 + j] = seen ? S[s][j] * scale_log2e : HX_NEG;
                     mx = fmaxf(mx, sc[s * 4 + j]);
                 }
@@ -340,7 +350,8 @@ extern "C" int ilm_attn_headmix_mfma(void* out, const void* qx, const void* kc, 
                                      const void* seg, const void* pos, const void* tiles, int n_tiles, const void* singles,
                                      int n_singles, const void* sink, int nh, int nkv, int d, int page, int max_blocks,
                                      int out_stride, float scale, int window, void* ws, int nz, int chunk_keys,
-                                     const void* seg_offsets, hipStream_t stream) {
+                                     const void* seg_offsets, int keep_first, hipStream_t stream) {
+    ILM_REQUIRE(keep_first >= 0, "attn_headmix_mfma: %d kept first tokens", keep_first);
     // single tokens whose heads come in groups of a multiple of 16: heads as the products' columns
     // (a block of 16 columns must lie in one key/value group: one group in all, or groups of a multiple of 16 heads)
     const bool hc = n_tiles == 0 && (nkv == 1 || (nh % 16 == 0 && (nh / (nkv > 0 ? nkv : 1)) % 16 == 0));
@@ -368,7 +379,7 @@ extern "C" int ilm_attn_headmix_mfma(void* out, const void* qx, const void* kc, 
                                          (const int*)block_tables, (const int*)seg, (const int*)pos, (const int*)tiles,    \
                                          n_tiles, (const int*)singles, (const float*)sink, nh, page, max_blocks,           \
                                          out_stride, scale_log2e, window, (float*)ws, chunk_keys,                          \
-                                         (const int*)seg_offsets);                                                         \
+                                         (const int*)seg_offsets, keep_first);                                             \
     }
 #define HX_BY_NC(D32_)                                                      \
     switch (nkv) {                                                          \

@@ -1,7 +1,7 @@
 // A feed-forward of many small experts of which every token uses a few.
 //
-//   ilm_moe_route     per token: the `top` largest of E router logits (ties to the lower index), their indices and
-//                     sigmoid(logit) as weights; one wave a token, all float32.
+//   ilm_moe_route     per token: the `top` largest of E router logits (ties to the lower index), their indices and as weights
+//                     a scale times sigmoid(logit) or the logit's softmax over all E experts; one wave a token, all float32.
 //   ilm_moe_sort      the (token, slot) pairs of a step ordered by expert: offsets per expert, the pair at every sorted
 //                     place and the place of every pair, and the list of row tiles (expert, first place, rows) that the
 //                     products below walk.  One block; the order inside an expert is whatever the atomics give, which no
@@ -9,10 +9,11 @@
 //   ilm_moe_gemm      for every tile of rows of one expert e: out[place] = f(W_e x[place]) with
 //                       GLU form    x = weight(pair) * h[token of the pair], W_e = [gate rows | up rows],
 //                                   g = min(gate, limit), u = clamp(up, -limit, limit), out = g sigmoid(alpha g) (u + 1)
-//                       plain form  x = rows in sorted order, out = W_e x
+//                       plain form  x = rows in sorted order (or, with the list of pairs, the pairs' token rows), out = W_e x
+//                                   or the square of relu(W_e x)
 //                     bfloat16 on v_mfma_f32_16x16x32_bf16 (tiles of 64 rows x 64 outputs, operands through LDS in steps of
 //                     64 k, the next step's loads in flight), float32 and odd sizes by FMA in ascending k.
-//   ilm_moe_combine   y[t] = sum over the token's slots of out[place of (t, slot)] (+ shared[t] * sigmoid(sg[t])).
+//   ilm_moe_combine   y[t] = sum over the token's slots of (weight of the pair *) out[place of (t, slot)] (+ shared[t] * sigmoid(sg[t])).
 //   ilm_glu_clamp     the experts' activation on fused [gate | up] rows of a dense product.
 #include "common.h"
 
@@ -31,7 +32,8 @@ __device__ __forceinline__ float moe_sigmoid(float v) { return 1.0f / (1.0f + ex
 
 // ---- routing -------------------------------------------------------------------------------------------------------
 __global__ void __launch_bounds__(256)
-moe_route_kernel(int* __restrict__ ids, float* __restrict__ wts, const float* __restrict__ z, int T_, int E, int top, int z_stride) {
+moe_route_kernel(int* __restrict__ ids, float* __restrict__ wts, const float* __restrict__ z, int T_, int E, int top, int z_stride,
+                 int softmax, float wscale) {
     const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (t >= T_) return;
     float v[MOE_MAX_E / 64];
@@ -39,6 +41,17 @@ moe_route_kernel(int* __restrict__ ids, float* __restrict__ wts, const float* __
     for (int i = 0; i < MOE_MAX_E / 64; ++i) {
         const int e = lane + 64 * i;
         v[i] = e < E ? z[(size_t)t * z_stride + e] : -INFINITY;
+    }
+    // softmax weights: the row's maximum and the sum of exponentials over all experts, in lane order
+    float zmax = -INFINITY, zsum = 0.f;
+    if (softmax) {
+#pragma unroll
+        for (int i = 0; i < MOE_MAX_E / 64; ++i) zmax = fmaxf(zmax, v[i]);
+        zmax = wave_max(zmax);
+#pragma unroll
+        for (int i = 0; i < MOE_MAX_E / 64; ++i)
+            if (lane + 64 * i < E) zsum += expf(v[i] - zmax);
+        zsum = wave_sum(zsum);
     }
     for (int s = 0; s < top; ++s) {
         float best = -INFINITY;
@@ -63,7 +76,7 @@ moe_route_kernel(int* __restrict__ ids, float* __restrict__ wts, const float* __
         if (bi >= E) bi = s;       // nothing compared larger (a row of NaNs): any valid expert, so that no index downstream is unset
         if (lane == 0) {
             ids[(size_t)t * top + s] = bi;
-            wts[(size_t)t * top + s] = moe_sigmoid(best);
+            wts[(size_t)t * top + s] = wscale * (softmax ? expf(best - zmax) / zsum : moe_sigmoid(best));
         }
 #pragma unroll
         for (int i = 0; i < MOE_MAX_E / 64; ++i)
@@ -71,10 +84,11 @@ moe_route_kernel(int* __restrict__ ids, float* __restrict__ wts, const float* __
     }
 }
 
-extern "C" int ilm_moe_route(void* ids, void* wts, const void* z, int T_, int E, int top, int z_stride, hipStream_t stream) {
+extern "C" int ilm_moe_route(void* ids, void* wts, const void* z, int T_, int E, int top, int z_stride, int softmax, float wscale,
+                             hipStream_t stream) {
     ILM_REQUIRE(T_ > 0 && E > 0 && E <= MOE_MAX_E && top > 0 && top <= E, "moe_route: %d tokens, %d experts (at most %d), top %d", T_, E,
                 MOE_MAX_E, top);
-    moe_route_kernel<<<(T_ + 3) / 4, 256, 0, stream>>>((int*)ids, (float*)wts, (const float*)z, T_, E, top, z_stride);
+    moe_route_kernel<<<(T_ + 3) / 4, 256, 0, stream>>>((int*)ids, (float*)wts, (const float*)z, T_, E, top, z_stride, softmax, wscale);
     ILM_LAUNCH_CHECK("moe_route");
     return 0;
 }
@@ -161,7 +175,7 @@ template <bool GLU>
 __global__ void __launch_bounds__(256)
 moe_gemm_mfma_kernel(bf16* __restrict__ out, int ld_out, const bf16* __restrict__ X, int ldx, const int* __restrict__ perm, int top,
                      const float* __restrict__ pair_w, const bf16* __restrict__ W, size_t w_expert, int ldw, const int* __restrict__ tiles,
-                     const int* __restrict__ n_tiles, int N, int K, float limit, float alpha) {
+                     const int* __restrict__ n_tiles, int N, int K, float limit, float alpha, int act) {
     constexpr int WR = GLU ? 2 : 1;
     __shared__ __attribute__((aligned(16))) bf16 xs[MOE_TM * MOE_LD];
     __shared__ __attribute__((aligned(16))) bf16 ws[WR * MOE_TN * MOE_LD];
@@ -175,7 +189,7 @@ moe_gemm_mfma_kernel(bf16* __restrict__ out, int ld_out, const bf16* __restrict_
         int row = -1;
         float w = 1.0f;
         if (tid < rows) {
-            if (GLU) {
+            if (GLU || perm != nullptr) {     // rows gathered from the tokens' rows (the plain form: only with a list of pairs)
                 const int pair = perm != nullptr ? perm[place0 + tid] : place0 + tid;
                 row = pair / top;
                 if (pair_w != nullptr) w = pair_w[pair];
@@ -268,6 +282,7 @@ moe_gemm_mfma_kernel(bf16* __restrict__ out, int ld_out, const bf16* __restrict_
             if (n < N) {
                 float v = acc[0][g][i];
                 if (GLU) v = moe_glu(v, acc[WR - 1][g][i], limit, alpha);
+                else if (act == 1) { v = fmaxf(v, 0.f); v *= v; }
                 orow[n] = from_f32<bf16>(v);
             }
         }
@@ -284,7 +299,7 @@ template <bool GLU, int WN>
 __global__ void __launch_bounds__(128 * WN) __attribute__((amdgpu_waves_per_eu(3, 3)))
 moe_gemm_mfma128_kernel(bf16* __restrict__ out, int ld_out, const bf16* __restrict__ X, int ldx, const int* __restrict__ perm, int top,
                         const float* __restrict__ pair_w, const bf16* __restrict__ W, size_t w_expert, int ldw, const int* __restrict__ tiles,
-                        const int* __restrict__ n_tiles, int N, int K, float limit, float alpha, int n_slices) {
+                        const int* __restrict__ n_tiles, int N, int K, float limit, float alpha, int act, int n_slices) {
     constexpr int THREADS = 128 * WN, RSTEP = THREADS / 8, XL = MOE_BM / RSTEP, WROWS = 64 * WN, WL = WROWS / RSTEP, HALF = 32 * WN;
     constexpr int TN = GLU ? HALF : WROWS;
     __shared__ __attribute__((aligned(16))) bf16 xs[MOE_BM * MOE_LD];
@@ -307,7 +322,7 @@ moe_gemm_mfma128_kernel(bf16* __restrict__ out, int ld_out, const bf16* __restri
         int row = -1;
         float w = 1.0f;
         if (tid < rows) {
-            if (GLU) {
+            if (GLU || perm != nullptr) {     // rows gathered from the tokens' rows (the plain form: only with a list of pairs)
                 const int pair = perm != nullptr ? perm[place0 + tid] : place0 + tid;
                 row = pair / top;
                 if (pair_w != nullptr) w = pair_w[pair];
@@ -426,6 +441,7 @@ moe_gemm_mfma128_kernel(bf16* __restrict__ out, int ld_out, const bf16* __restri
                 if (nb + i < N) {
                     float v = acc[f][g][i];
                     if (GLU) v = moe_glu(sw * v, sw * acc[f + 2][g][i], limit, alpha);
+                    else if (act == 1) { v = fmaxf(v, 0.f); v *= v; }
                     orow[nb + i] = from_f32<bf16>(v);
                 }
             }
@@ -439,7 +455,7 @@ template <typename T, bool GLU>
 __global__ void __launch_bounds__(256)
 moe_gemm_plain_kernel(T* __restrict__ out, int ld_out, const T* __restrict__ X, int ldx, const int* __restrict__ perm, int top,
                       const float* __restrict__ pair_w, const T* __restrict__ W, size_t w_expert, int ldw, const int* __restrict__ tiles,
-                      const int* __restrict__ n_tiles, int N, int K, float limit, float alpha) {
+                      const int* __restrict__ n_tiles, int N, int K, float limit, float alpha, int act) {
     constexpr int WR = GLU ? 2 : 1;
     constexpr int KS = 16;
     __shared__ float xs[KS][MOE_TM + 1];
@@ -454,7 +470,7 @@ moe_gemm_plain_kernel(T* __restrict__ out, int ld_out, const T* __restrict__ X, 
         int row = -1;
         float w = 1.0f;
         if (tid < rows) {
-            if (GLU) {
+            if (GLU || perm != nullptr) {     // rows gathered from the tokens' rows (the plain form: only with a list of pairs)
                 const int pair = perm != nullptr ? perm[place0 + tid] : place0 + tid;
                 row = pair / top;
                 if (pair_w != nullptr) w = pair_w[pair];
@@ -515,6 +531,7 @@ moe_gemm_plain_kernel(T* __restrict__ out, int ld_out, const T* __restrict__ X, 
             if (n < N) {
                 float v = acc[0][a][b];
                 if (GLU) v = moe_glu(v, acc[WR - 1][a][b], limit, alpha);
+                else if (act == 1) { v = fmaxf(v, 0.f); v *= v; }
                 out[(size_t)(place0 + m) * ld_out + n] = from_f32<T>(v);
             }
         }
@@ -523,13 +540,14 @@ moe_gemm_plain_kernel(T* __restrict__ out, int ld_out, const T* __restrict__ X, 
 
 extern "C" int ilm_moe_gemm(void* out, int ld_out, const void* X, int ldx, const void* perm, int top, const void* pair_w, const void* W,
                             long w_expert, int ldw, const void* tiles, const void* n_tiles, int max_tiles, int N, int K, int glu,
-                            float limit, float alpha, int dtype, int force_plain, int tile_rows, int wide_mode, hipStream_t stream) {
+                            float limit, float alpha, int act, int dtype, int force_plain, int tile_rows, int wide_mode, hipStream_t stream) {
+    ILM_REQUIRE(act == 0 || (act == 1 && !glu), "moe_gemm: activation %d (0: none, 1: the square of relu, in the plain form)", act);
     ILM_REQUIRE(tile_rows == MOE_TM || tile_rows == MOE_BM, "moe_gemm: tiles of %d rows (%d or %d)", tile_rows, MOE_TM, MOE_BM);
     ILM_REQUIRE(max_tiles > 0 && max_tiles <= 65535 && N > 0 && K > 0 && top > 0, "moe_gemm: bad sizes (tiles %d, N %d, K %d)", max_tiles, N, K);
     ILM_REQUIRE(ld_out >= N && ldx >= K && ldw >= K, "moe_gemm: rows shorter than their products");
     dim3 grid((N + MOE_TN - 1) / MOE_TN, max_tiles);
 #define MOE_ARGS(T__) (T__*)out, ld_out, (const T__*)X, ldx, (const int*)perm, top, (const float*)pair_w, (const T__*)W, (size_t)w_expert, ldw, \
-                      (const int*)tiles, (const int*)n_tiles, N, K, limit, alpha
+                      (const int*)tiles, (const int*)n_tiles, N, K, limit, alpha, act
     const bool aligned = K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && w_expert % 8 == 0 && ((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0;
     if (dtype == ILM_DTYPE_BF16 && aligned && !force_plain && tile_rows == MOE_BM) {
         // 256 rows of W a tile on demand (wide_mode 1) where the outputs fill one: a third fewer bytes a product from the caches, and
@@ -565,26 +583,30 @@ extern "C" int ilm_moe_gemm(void* out, int ld_out, const void* X, int ldx, const
 // ---- the sum over a token's experts --------------------------------------------------------------------------------
 template <typename T>
 __global__ void moe_combine_kernel(T* __restrict__ y, const T* __restrict__ pair_out, const int* __restrict__ inv, int top,
-                                   const T* __restrict__ shared, const float* __restrict__ sg, int sg_stride, int H, int ld_pair) {
+                                   const T* __restrict__ shared, const float* __restrict__ sg, int sg_stride, int H, int ld_pair,
+                                   const float* __restrict__ pair_w) {
     const int t = blockIdx.x;
     const float gate = sg != nullptr ? moe_sigmoid(sg[(size_t)t * sg_stride]) : 1.0f;
     for (int j = threadIdx.x; j < H; j += blockDim.x) {
         float v = 0.f;
-        for (int s = 0; s < top; ++s) v += to_f32(pair_out[(size_t)inv[(size_t)t * top + s] * ld_pair + j]);
+        for (int s = 0; s < top; ++s) {
+            const float o = to_f32(pair_out[(size_t)inv[(size_t)t * top + s] * ld_pair + j]);
+            v = pair_w != nullptr ? fmaf(pair_w[(size_t)t * top + s], o, v) : v + o;
+        }
         if (shared != nullptr) v = fmaf(to_f32(shared[(size_t)t * H + j]), gate, v);
         y[(size_t)t * H + j] = from_f32<T>(v);
     }
 }
 
 extern "C" int ilm_moe_combine(void* y, const void* pair_out, const void* inv, int top, const void* shared, const void* sg, int sg_stride,
-                               int T_, int H, int ld_pair, int dtype, hipStream_t stream) {
+                               int T_, int H, int ld_pair, const void* pair_w, int dtype, hipStream_t stream) {
     ILM_REQUIRE(T_ > 0 && H > 0 && top > 0 && ld_pair >= H, "moe_combine: bad sizes");
     if (dtype == ILM_DTYPE_F32)
         moe_combine_kernel<float><<<T_, 256, 0, stream>>>((float*)y, (const float*)pair_out, (const int*)inv, top, (const float*)shared,
-                                                          (const float*)sg, sg_stride, H, ld_pair);
+                                                          (const float*)sg, sg_stride, H, ld_pair, (const float*)pair_w);
     else if (dtype == ILM_DTYPE_BF16)
         moe_combine_kernel<bf16><<<T_, 256, 0, stream>>>((bf16*)y, (const bf16*)pair_out, (const int*)inv, top, (const bf16*)shared,
-                                                         (const float*)sg, sg_stride, H, ld_pair);
+                                                         (const float*)sg, sg_stride, H, ld_pair, (const float*)pair_w);
     else
         ILM_REQUIRE(false, "moe_combine: unknown dtype %d", dtype);
     ILM_LAUNCH_CHECK("moe_combine");

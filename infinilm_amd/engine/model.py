@@ -14,6 +14,7 @@ from typing import Dict, List
 import torch
 
 from .. import kernels
+from ..cache.manager import Lent
 from ..config.spec import ModelSpec, PartSpec
 from ..parts import BuildContext, Param, ResidualStream, build_block
 from ..parts.base import join_name
@@ -57,6 +58,12 @@ class CausalLM:
                 if need != self.cache_needs[run.cache]:
                     raise ValueError(f"layer {run.layer} reads cache entry {run.cache}, whose writer keeps "
                                      f"{self.cache_needs[run.cache]}, but needs {need}")
+        for run in spec.order:
+            if run.borrows is not None:
+                want = getattr(self.blocks[run.layer].mixer, "borrowed_need", lambda: None)()
+                held = self.cache_needs[run.borrows]
+                if want is None or want not in (held if isinstance(held, (tuple, list)) else (held,)):
+                    raise ValueError(f"layer {run.layer} borrows cache entry {run.borrows}, which keeps {held}, but reads {want}")
 
     # ---- tensors by checkpoint name ---------------------------------------------------------
     @property
@@ -124,6 +131,8 @@ class CausalLM:
                 if run.start.vector_row is not None:
                     stream.push_more(self.run_vectors[run.start.vector_row], 1.0)
             view = cache.view(run.cache, batch, run.writes_cache) if run.cache is not None else None
+            if run.borrows is not None:
+                view = Lent(view, cache.view(run.borrows, batch, False))
             self.blocks[run.layer].forward(stream, batch, view)
             if taps is not None:
                 stream.settle()

@@ -117,7 +117,8 @@ class Scheduler:
         longest portion of a step, and the page in which the window's edge lies."""
         pages = self._pages_for(n_tokens)
         if group.window > 0:
-            pages = min(pages, self._pages_for(group.window + min(self.chunk_size, self.max_num_batched_tokens)) + 1)
+            pages = min(pages, self._pages_for(group.window + min(self.chunk_size, self.max_num_batched_tokens)) + 1
+                        + self._pages_for(getattr(group, "keep_first", 0)))
         return pages
 
     def _worst_case_pages(self, req: InferenceRequest) -> List[int]:

@@ -1365,8 +1365,10 @@ def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                       seg_of_token: torch.Tensor, positions: torch.Tensor, nh: int, nkv: int, d: int, dv: int, scale: float,
                       window: int = 0, mix: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None,
                       tiles: Optional[torch.Tensor] = None, single_rows: Optional[torch.Tensor] = None,
-                      max_total_len: Optional[int] = None, seg_offsets: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Attention of every token over its request's cached keys (its last `window` positions, or all) where the scaled
+                      max_total_len: Optional[int] = None, seg_offsets: Optional[torch.Tensor] = None,
+                      keep_first: int = 0) -> torch.Tensor:
+    """Attention of every token over its request's cached keys (its last `window` positions, or all; with `keep_first` the
+    sequence's first that many keys stay seen however far the window has moved) where the scaled
     scores of the heads are mixed before the softmax, s_h = sum_g mix[h, g] raw_g (`mix` float32 [nh, nh] or None),
     and every head's denominator holds one more term exp(sink[h]) (`sink` float32 [nh] or None); with neither it is the
     attention of `paged_attention` with its weights kept in float32 up to the second product.  q, caches, block
@@ -1435,11 +1437,137 @@ def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         _run("ilm_attn_headmix_mfma", out.data_ptr(), qx.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
              seg_of_token.data_ptr(), positions.data_ptr(), _ptr(tiles) if n_tiles else None, n_tiles, _ptr(rows), n_single,
              _ptr(sink), nh, nkv, d, page, block_tables.shape[1], out.stride(0), float(scale), int(window), _ptr(ws), nz, chunk,
-             _ptr(seg_offsets) if n_tiles else None, _stream(), label="ilm_attn_headmix_mfma (unmixed)" if mix is None and sink is None else None)
+             _ptr(seg_offsets) if n_tiles else None, int(keep_first), _stream(),
+             label="ilm_attn_headmix_mfma (unmixed)" if mix is None and sink is None else None)
         return out
     _run("ilm_attn_headmix", out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
          seg_of_token.data_ptr(), positions.data_ptr(), None, T, _ptr(mix), _ptr(sink), nh, nkv, d, int(dv), page,
-         block_tables.shape[1], q.stride(0), out.stride(0), float(scale), int(window), _dt(q), _stream())
+         block_tables.shape[1], q.stride(0), out.stride(0), float(scale), int(window), int(keep_first), _dt(q), _stream())
+    return out
+
+
+# ---- attention in maps over shared values ("differential" attention) ---------------------------------------------------
+def maps_norm_rope_kvwrite(src: torch.Tensor, q_off: int, k_off: int, v_off: int, positions: torch.Tensor,
+                           freq: Optional[torch.Tensor], q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
+                           k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], slots: Optional[torch.Tensor],
+                           heads: int, kv_heads: int, maps: int, dim: int, vdim: int, rd: int, eps: float,
+                           out_dtype: torch.dtype) -> torch.Tensor:
+    """From rows `src` (float32 or `out_dtype`) that hold [q: heads maps dim] at entry q_off, [k: kv_heads maps dim] at k_off
+    and [v: kv_heads vdim] at v_off (k_off < 0: no keys and values in these rows): every q and k unit of `dim` entries
+    RMS-normed times `q_weight` / `k_weight` [dim] (None: no norm) and its first `rd` entries turned in the pairs (i, i + rd/2)
+    by position x freq[i]; k goes to the paged cache with a head's maps side by side (entry m dim + e of cache heads of d >=
+    maps dim), v to the value cache, at `slots` (None: no write).  Returns the queries [T, heads maps dim] as `out_dtype`."""
+    _dev(src, positions, freq, q_weight, k_weight, k_cache, v_cache, slots)
+    _rows(src, "src")
+    _i32(positions, "positions")
+    T = src.shape[0]
+    need = max(q_off + heads * maps * dim, (k_off + kv_heads * maps * dim) if k_off >= 0 else 0, (v_off + kv_heads * vdim) if k_off >= 0 else 0)
+    if src.shape[1] < need or positions.numel() != T or src.dtype not in (F32, out_dtype):
+        raise KernelError(f"rows of {src.shape[1]} ({src.dtype}) do not hold the queries, keys and values asked for")
+    if rd and (freq is None or freq.dtype != F32 or freq.numel() != rd // 2 or not freq.is_contiguous()):
+        raise KernelError(f"frequencies must be float32 [{rd // 2}]")
+    if k_off >= 0 and (q_weight is None) != (k_weight is None):
+        raise KernelError("a norm weight for q and k, or for neither")
+    for w in (q_weight, k_weight):
+        if w is not None and (tuple(w.shape) != (dim,) or not w.is_contiguous() or w.dtype != q_weight.dtype):
+            raise KernelError(f"a query/key norm weight must be [{dim}]")
+    page, d = 1, maps * dim
+    write = k_off >= 0 and slots is not None
+    if write:
+        _i32(slots, "slots")
+        if k_cache.dtype != out_dtype or slots.numel() != T:
+            raise KernelError("cache dtype or slots do not match the rows")
+        d = k_cache.shape[3]
+        page = _check_cache(k_cache, v_cache, kv_heads, d)
+    q = torch.empty((T, heads * maps * dim), dtype=out_dtype, device=src.device)
+    _run("ilm_maps_norm_rope_kvwrite", q.data_ptr(), src.data_ptr(), src.stride(0), int(q_off), int(k_off), int(v_off),
+         positions.data_ptr(), _ptr(freq), _ptr(q_weight), _ptr(k_weight), _ptr(k_cache) if write else None,
+         _ptr(v_cache) if write else None, _ptr(slots) if write else None, T, int(heads), int(kv_heads), int(maps), int(dim),
+         int(vdim), int(d), int(rd), float(eps), page, _dt(src), _DT[out_dtype], _dt(q_weight) if q_weight is not None else _DT[out_dtype],
+         _stream())
+    return q
+
+
+def maps_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                   seg_of_token: torch.Tensor, positions: torch.Tensor, heads: int, kv_heads: int, maps: int, dim: int, vdim: int,
+                   scale: float, window: int = 0, keep_first: int = 0, sink: Optional[torch.Tensor] = None,
+                   lambda_vectors=None, diff: float = 0.0, norm_eps: float = -1.0, out_scale: float = 1.0) -> torch.Tensor:
+    """Every query head's `maps` softmax attentions over its request's cached keys (the last `window` positions and the first
+    `keep_first`, or all), each map against its own part of the key head (entries m dim ..) and all over the same values;
+    `sink` float32 [heads]: one more term exp(sink_h) in the denominators.  One map: the attention's result.  Two maps:
+    a_0 - lambda a_1 with lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff from `lambda_vectors` = (lq1, lk1, lq2, lk2), each [dim];
+    then, with norm_eps >= 0, divided by its root mean square over the head's vdim entries; times out_scale.  All sums and
+    weights float32.  q [T, heads maps dim] dense; returns [T, heads vdim]."""
+    _dev(q, k_cache, v_cache, block_tables, seg_of_token, positions, sink)
+    _i32(block_tables, "block_tables")
+    _i32(seg_of_token, "seg_of_token")
+    _i32(positions, "positions")
+    T = q.shape[0]
+    if not q.is_contiguous() or q.shape[1] != heads * maps * dim:
+        raise KernelError(f"queries must be dense rows of {heads} x {maps} x {dim}")
+    if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
+        raise KernelError(f"cache dtype {k_cache.dtype} differs from the activations' {q.dtype}")
+    d = k_cache.shape[3] if k_cache.dim() == 4 else 0
+    page = _check_cache(k_cache, v_cache, kv_heads, d)
+    if seg_of_token.numel() != T or positions.numel() != T or block_tables.dim() != 2:
+        raise KernelError("per-token metadata does not match the number of tokens")
+    if sink is not None and (sink.dtype != F32 or tuple(sink.shape) != (heads,) or not sink.is_contiguous()):
+        raise KernelError(f"the denominators' extra terms must be contiguous float32 [{heads}]")
+    lv = [None] * 4
+    if maps == 2:
+        if lambda_vectors is None or len(lambda_vectors) != 4:
+            raise KernelError("two maps need the four vectors of their weight")
+        lv = list(lambda_vectors)
+        _dev(*lv)
+        for v in lv:
+            if tuple(v.shape) != (dim,) or not v.is_contiguous() or v.dtype != lv[0].dtype:
+                raise KernelError(f"the maps' weight vectors must be contiguous [{dim}] of one dtype")
+    out = torch.empty((T, heads * vdim), dtype=q.dtype, device=q.device)
+    _run("ilm_attn_maps", out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
+         seg_of_token.data_ptr(), positions.data_ptr(), None, T, int(heads), int(kv_heads), int(maps), int(dim), int(vdim), int(d),
+         page, block_tables.shape[1], out.stride(0), float(scale), int(window), int(keep_first), _ptr(sink), _ptr(lv[0]), _ptr(lv[1]),
+         _ptr(lv[2]), _ptr(lv[3]), float(diff), float(norm_eps), float(out_scale), _dt(q), _dt(lv[0]) if lv[0] is not None else _dt(q),
+         _stream())
+    return out
+
+
+# ---- a selective scan with a decay per channel and state entry -----------------------------------------------------------
+SELECTIVE_SCAN_MAX_STATE = 256   # most state entries a channel (ilm_selective_scan_max_state())
+
+
+def selective_scan(x: torch.Tensor, raw_dt: torch.Tensor, dt_bias: torch.Tensor, B: torch.Tensor, C: torch.Tensor, z: torch.Tensor,
+                   a_log: torch.Tensor, skip: torch.Tensor, pool: torch.Tensor, state_in: torch.Tensor, state_out: torch.Tensor,
+                   seg_offsets: torch.Tensor, segments: int) -> torch.Tensor:
+    """Per channel c and state entry n, token by token from the request's state row: dt = softplus(raw_dt + dt_bias),
+    S[c, n] <- exp(-exp(a_log[c, n]) dt_c) S[c, n] + dt_c x_c B_n, y_c = sum_n S[c, n] C_n + skip_c x_c, out = y silu(z).
+    x float32 [T, inner]; raw_dt, z [T, inner] and B, C [T, state] in the activations' dtype (views with dense rows; B and C of
+    one row stride); a_log float32 [inner, state], skip float32 [inner]; pool float32 [rows, inner, state].  Returns
+    [T, inner] in the activations' dtype."""
+    _dev(x, raw_dt, dt_bias, B, C, z, a_log, skip, pool, state_in, state_out, seg_offsets)
+    for t, nm in ((x, "x"), (raw_dt, "raw_dt"), (B, "B"), (C, "C"), (z, "z")):
+        _rows(t, nm)
+    T, inner = x.shape
+    state = B.shape[1]
+    dt = raw_dt.dtype
+    if x.dtype != F32 or raw_dt.shape != (T, inner) or z.shape != (T, inner) or z.dtype != dt or B.dtype != dt or C.dtype != dt \
+            or B.shape != (T, state) or C.shape != (T, state) or B.stride(0) != C.stride(0):
+        raise KernelError("the scan's operands do not fit each other")
+    if state > SELECTIVE_SCAN_MAX_STATE:
+        raise KernelError(f"{state} state entries a channel (at most {SELECTIVE_SCAN_MAX_STATE})")
+    if a_log.dtype != F32 or tuple(a_log.shape) != (inner, state) or not a_log.is_contiguous() or skip.dtype != F32 \
+            or tuple(skip.shape) != (inner,) or tuple(dt_bias.shape) != (inner,) or not dt_bias.is_contiguous():
+        raise KernelError(f"a_log float32 [{inner}, {state}], skip float32 [{inner}], dt_bias [{inner}]")
+    if pool.dtype != F32 or not pool.is_contiguous() or tuple(pool.shape[1:]) != (inner, state):
+        raise KernelError(f"the state pool must be float32 [rows, {inner}, {state}], got {tuple(pool.shape)}")
+    for t, nm in ((state_in, "state_in"), (state_out, "state_out"), (seg_offsets, "seg_offsets")):
+        _i32(t, nm)
+    if state_in.numel() < segments or state_out.numel() < segments or seg_offsets.numel() < segments + 1:
+        raise KernelError("state rows and offsets must cover every segment")
+    out = torch.empty((T, inner), dtype=dt, device=x.device)
+    _run("ilm_selective_scan", out.data_ptr(), out.stride(0), x.data_ptr(), x.stride(0), raw_dt.data_ptr(), raw_dt.stride(0),
+         dt_bias.data_ptr(), B.data_ptr(), C.data_ptr(), B.stride(0), z.data_ptr(), z.stride(0), a_log.data_ptr(), skip.data_ptr(),
+         pool.data_ptr(), state_in.data_ptr(), state_out.data_ptr(), seg_offsets.data_ptr(), int(segments), inner, state, _DT[dt],
+         _dt(dt_bias), _stream())
     return out
 
 
@@ -1614,9 +1742,11 @@ class ExpertPlan:
     __slots__ = ("ids", "weights", "perm", "inv", "tiles", "n_tiles", "offsets", "max_tiles", "top", "pairs", "tile_rows")
 
 
-def moe_route(logits: torch.Tensor, experts: int, top: int, big_tiles_ok: bool = False) -> ExpertPlan:
+def moe_route(logits: torch.Tensor, experts: int, top: int, big_tiles_ok: bool = False, softmax: bool = False,
+              weight_scale: float = 1.0) -> ExpertPlan:
     """From float32 router logits [T, >= experts] (the first `experts` entries of a row count): the `top` experts of every token
-    with sigmoid(logit) as their weights, and the pairs ordered by expert for `moe_gemm`.  `big_tiles_ok`: the products that
+    with weight_scale x sigmoid(logit) (or, `softmax`, weight_scale x the logit's softmax over all experts) as their weights, and
+    the pairs ordered by expert for `moe_gemm`.  `big_tiles_ok`: the products that
     follow are bfloat16 with every K a multiple of 8, so a step of many pairs an expert may be cut into tiles of 128 rows."""
     _dev(logits)
     if logits.dtype != F32 or logits.dim() != 2 or logits.stride(1) != 1 or logits.shape[1] < experts:
@@ -1628,7 +1758,8 @@ def moe_route(logits: torch.Tensor, experts: int, top: int, big_tiles_ok: bool =
     plan.top, plan.pairs = int(top), P
     plan.ids = torch.empty((T, top), dtype=torch.int32, device=dev)
     plan.weights = torch.empty((T, top), dtype=F32, device=dev)
-    _run("ilm_moe_route", plan.ids.data_ptr(), plan.weights.data_ptr(), logits.data_ptr(), T, int(experts), int(top), logits.stride(0), _stream())
+    _run("ilm_moe_route", plan.ids.data_ptr(), plan.weights.data_ptr(), logits.data_ptr(), T, int(experts), int(top), logits.stride(0),
+         int(bool(softmax)), float(weight_scale), _stream())
     plan.tile_rows = MOE_BIG_TILE_ROWS if big_tiles_ok and not MOE_FORCE_PLAIN and P >= MOE_BIG_MIN_ROWS * experts else MOE_TILE_ROWS
     plan.max_tiles = min(P, P // plan.tile_rows + min(experts, P))
     book = torch.empty((experts + 1 + 2 * P + 3 * plan.max_tiles + 1,), dtype=torch.int32, device=dev)
@@ -1642,30 +1773,36 @@ def moe_route(logits: torch.Tensor, experts: int, top: int, big_tiles_ok: bool =
     return plan
 
 
-def moe_gemm(x: torch.Tensor, w: torch.Tensor, plan: ExpertPlan, glu: bool, limit: float = 0.0, alpha: float = 1.702) -> torch.Tensor:
+def moe_gemm(x: torch.Tensor, w: torch.Tensor, plan: ExpertPlan, glu: bool, limit: float = 0.0, alpha: float = 1.702,
+             gather: bool = False, act: str = "none") -> torch.Tensor:
     """The experts' products over the ordered pairs.  `glu`: x [T, K] are the tokens' rows, w [E, 2 I, K] holds every expert's
     gate rows and then its up rows; a pair's row is its token's row times the pair's weight, and the result [pairs, I] is
     min(gate, limit) * sigmoid(alpha * min(gate, limit)) * (clamp(up, -limit, limit) + 1) in sorted order.  Otherwise x [pairs, K] are rows
-    in sorted order and w [E, N, K]: the result is [pairs, N] in sorted order."""
+    in sorted order (`gather`: the tokens' rows [T, K], from which every pair takes its token's, unweighted) and w [E, N, K]: the
+    result is [pairs, N] in sorted order, `act` ("none" or "relu2", the square of relu) applied to it."""
     _dev(x, w)
     _rows(x, "x")
     E, Nw, K = w.shape
     if not w.is_contiguous() or w.dtype != x.dtype or x.shape[1] != K or (glu and Nw % 2):
         raise KernelError(f"experts of shape {tuple(w.shape)} do not fit rows of {tuple(x.shape)}")
     N = Nw // 2 if glu else Nw
-    if not glu and x.shape[0] != plan.pairs:
+    if not glu and not gather and x.shape[0] != plan.pairs:
         raise KernelError("rows in sorted order: one a pair")
+    if act not in ("none", "relu2") or (glu and act != "none"):
+        raise KernelError(f"the experts' plain product takes no activation or relu2, got {act!r}")
     out = torch.empty((plan.pairs, N), dtype=x.dtype, device=x.device)
-    _run("ilm_moe_gemm", out.data_ptr(), N, x.data_ptr(), x.stride(0), plan.perm.data_ptr(), plan.top, plan.weights.data_ptr() if glu else None,
+    _run("ilm_moe_gemm", out.data_ptr(), N, x.data_ptr(), x.stride(0), plan.perm.data_ptr() if (glu or gather) else None, plan.top,
+         plan.weights.data_ptr() if glu else None,
          w.data_ptr(), Nw * K, K, plan.tiles.data_ptr(), plan.n_tiles.data_ptr(), plan.max_tiles, N, K, int(bool(glu)), float(limit),
-         float(alpha), _dt(x), int(MOE_FORCE_PLAIN), plan.tile_rows, int(MOE_WIDE), _stream(), label="ilm_moe_gemm (gate/up)" if glu else "ilm_moe_gemm (down)")
+         float(alpha), 1 if act == "relu2" else 0, _dt(x), int(MOE_FORCE_PLAIN), plan.tile_rows, int(MOE_WIDE), _stream(), label="ilm_moe_gemm (gate/up)" if glu else "ilm_moe_gemm (down)")
     return out
 
 
 def moe_combine(pair_out: torch.Tensor, plan: ExpertPlan, shared: Optional[torch.Tensor] = None,
-                shared_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """y[t] = sum over the token's slots of pair_out[place of (t, slot)] + shared[t] * sigmoid(shared_gate[t]); `shared_gate` is a
-    float32 column (one number a token, any stride)."""
+                shared_gate: Optional[torch.Tensor] = None, weighted: bool = False) -> torch.Tensor:
+    """y[t] = sum over the token's slots of pair_out[place of (t, slot)] (`weighted`: times the pair's weight of the plan, in
+    float32) + shared[t] * sigmoid(shared_gate[t]); `shared_gate` is a float32 column (one number a token, any stride; None: the
+    shared rows are added as they are)."""
     _dev(pair_out, shared, shared_gate)
     _rows(pair_out, "pair_out")
     P, H = pair_out.shape
@@ -1682,7 +1819,8 @@ def moe_combine(pair_out: torch.Tensor, plan: ExpertPlan, shared: Optional[torch
             sg_stride = shared_gate.stride(0)
     out = torch.empty((T, H), dtype=pair_out.dtype, device=pair_out.device)
     _run("ilm_moe_combine", out.data_ptr(), pair_out.data_ptr(), plan.inv.data_ptr(), plan.top, _ptr(shared),
-         _ptr(shared_gate) if shared is not None else None, sg_stride, T, H, pair_out.stride(0), _dt(pair_out), _stream())
+         _ptr(shared_gate) if shared is not None else None, sg_stride, T, H, pair_out.stride(0),
+         plan.weights.data_ptr() if weighted else None, _dt(pair_out), _stream())
     return out
 
 

@@ -1,1 +1,1 @@
-from . import kekevik, minicpm4, patadra, pugavik  # noqa: F401
+from . import bebuzen, kekevik, minicpm4, patadra, pugavik  # noqa: F401

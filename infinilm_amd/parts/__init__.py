@@ -1,4 +1,4 @@
-from . import (attention, block, ends, latent_attention, linear_attention, mlp, moe, norm, parallel, rotary, side_input, state_space,  # noqa: F401
+from . import (attention, block, differential_attention, ends, latent_attention, linear_attention, mlp, moe, norm, parallel, rotary, selective_scan, side_input, state_space,  # noqa: F401
                temperature)   # (register the built-in kinds)
 from .base import (BuildContext, FeedForward, Mixer, Norm, Param, Part, PositionEncoding, ResidualStream)
 from .block import build_block

@@ -42,7 +42,8 @@ class GQAttention(Mixer):
                  value_dim: Optional[int] = None, softcap: float = 0.0,
                  names: Sequence[str] = ("q_proj", "k_proj", "v_proj", "o_proj"), suffix: str = "weight",
                  whole_output: bool = False, head_mix: bool = False, sink: bool = False,
-                 mix_names: Sequence[str] = ("head_mix", "sink"), position_prefix: str = "position", bias_suffix: str = "bias"):
+                 mix_names: Sequence[str] = ("head_mix", "sink"), position_prefix: str = "position", bias_suffix: str = "bias",
+                 keep_first: int = 0, fixed_sink: Optional[float] = None):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads do not divide into {num_kv_heads} groups")
         self.nh, self.nkv = int(num_heads), int(num_kv_heads)
@@ -64,6 +65,17 @@ class GQAttention(Mixer):
         self.mix_names = tuple(mix_names)
         self.head_mix = torch.empty((self.nh, self.nh), dtype=torch.float32, device=ctx.device) if head_mix else None
         self.sink = torch.empty((self.nh,), dtype=torch.float32, device=ctx.device) if sink else None
+        # `fixed_sink`: the denominators' extra term is exp(fixed_sink) for every head, a constant of the design and no tensor
+        # of a checkpoint (0.0: one is added to every denominator); `keep_first`: with a window, the sequence's first
+        # that many tokens stay seen at their true positions however far the window has moved
+        self.fixed_sink = None
+        if fixed_sink is not None:
+            if sink:
+                raise ValueError("the denominators' extra term is learned or fixed, not both")
+            self.fixed_sink = torch.full((self.nh,), float(fixed_sink), dtype=torch.float32, device=ctx.device)
+        self.keep_first = int(keep_first) if self.window > 0 else 0
+        if self.keep_first < 0:
+            raise ValueError(f"{keep_first} kept first tokens")
         if getattr(self.position, "head_dim", self.d) not in (0, self.d):
             raise ValueError(f"the position encoding is made for heads of {self.position.head_dim}, the mixer's have {self.d}")
 
@@ -79,7 +91,7 @@ class GQAttention(Mixer):
         return out
 
     def cache_need(self):
-        return PagedKV(self.nkv, self.d, self.window)
+        return PagedKV(self.nkv, self.d, self.window, self.keep_first)
 
     takes_tail = True
     records_mixed_steps = True
@@ -99,14 +111,15 @@ class GQAttention(Mixer):
             pe.encode_and_store(qkv, batch, cache_view, self.nh, self.nkv, self.d)
             if batch.taps is not None:
                 batch.taps.setdefault("qkv_rotated", []).append(qkv.clone())
-        if self.head_mix is not None or self.sink is not None:
+        sink = self.sink if self.sink is not None else self.fixed_sink
+        if self.head_mix is not None or sink is not None or self.keep_first:
             if self.softcap:
                 raise ValueError("scores mixed over the heads take no cap")
             o = kernels.headmix_attention(qkv, cache_view.k, cache_view.v, cache_view.block_tables, batch.seg_of_token,
                                           batch.positions, self.nh, self.nkv, self.d, self.dv, self.scale, self.window,
-                                          mix=self.head_mix, sink=self.sink, tiles=batch.att_tiles,
+                                          mix=self.head_mix, sink=sink, tiles=batch.att_tiles,
                                           single_rows=batch.att_single_rows, max_total_len=batch.max_total_len,
-                                          seg_offsets=batch.seg_offsets)
+                                          seg_offsets=batch.seg_offsets, keep_first=self.keep_first)
         else:
             o = self._plain_attention(qkv, batch, cache_view)
         if tail is not None:   # the output projection adds into the residual stream itself, where its kernel can

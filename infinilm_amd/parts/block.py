@@ -226,6 +226,48 @@ class GatedPreNormBlock:
             self.side.forward(stream, batch)
 
 
+@register_arrangement("branch_norm")
+class BranchNormBlock:
+    """x += s * norm1(mixer(x)); x += s * norm2(ffn(x)): the sublayers read the residual stream itself (its rows in the
+    activations' dtype), and the only norms stand on the sublayers' outputs.  A layer may have no feed-forward (then no
+    `ffn` and no `norm2`).  A sublayer's output is left with the stream together with its norm (`push_normed`); the kernel that
+    next reads the stream norms it, adds it and hands out the rows (`ResidualStream.rows`), in one pass."""
+
+    def __init__(self, spec: LayerSpec, ctx: BuildContext):
+        self.spec = spec
+        self.slots = tuple(s for s in ("mixer", "norm1", "ffn", "norm2") if s in spec.parts)
+        if not {"mixer", "norm1"} <= set(self.slots) or (("ffn" in self.slots) != ("norm2" in self.slots)):
+            raise ValueError(f"layer {spec.prefix}: a layer with normed branches has mixer, norm1 and, with a feed-forward, norm2")
+        self.mixer = build_mixer(spec.parts["mixer"], ctx)
+        self.norm1 = build_norm(spec.parts["norm1"], ctx)
+        self.ffn = build_feed_forward(spec.parts["ffn"], ctx) if "ffn" in self.slots else None
+        self.norm2 = build_norm(spec.parts["norm2"], ctx) if "ffn" in self.slots else None
+        self.residual_scale = float(spec.residual_scale)
+        self.dtype = ctx.dtype
+
+    def named_parameters(self) -> Dict[str, Param]:
+        out: Dict[str, Param] = {}
+        for slot in self.slots:
+            for name, p in getattr(self, slot).named_parameters().items():
+                out[join_name(self.spec.prefix, self.spec.names[slot], name)] = p
+        return out
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    @property
+    def records_mixed_steps(self) -> bool:
+        return bool(getattr(self.mixer, "records_mixed_steps", False)
+                    and (self.ffn is None or getattr(self.ffn, "records_mixed_steps", False)))
+
+    def forward(self, stream: ResidualStream, batch, cache_view) -> None:
+        y = self.mixer.forward(stream.rows(self.dtype), batch, cache_view)
+        stream.push_normed(y, self.norm1, self.residual_scale)
+        if self.ffn is not None:
+            y = self.ffn.forward(stream.rows(self.dtype), batch)
+            stream.push_normed(y, self.norm2, self.residual_scale)
+
+
 def build_block(spec: LayerSpec, ctx: BuildContext):
     try:
         cls = ARRANGEMENTS[spec.arrangement]

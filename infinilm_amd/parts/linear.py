@@ -37,8 +37,8 @@ class FusedLinear:
         for size, oh in zip(self.out_sizes, self.out_heads):
             if oh is not None and (oh[0] * oh[2] != size or oh[1] > oh[2]):
                 raise ValueError(f"{oh[0]} heads of {oh[1]} filled up to {oh[2]} are not {size} rows")
-        if self.in_heads is not None and (self.in_heads[0] * self.in_heads[2] != self.in_features or bias):
-            raise ValueError("filled-up columns must make up the whole input (and take no bias)")
+        if self.in_heads is not None and self.in_heads[0] * self.in_heads[2] != self.in_features:
+            raise ValueError("filled-up columns must make up the whole input")
         n = sum(self.out_sizes)
         padded = self.in_heads is not None or any(oh is not None and oh[1] != oh[2] for oh in self.out_heads)
         make = torch.zeros if padded else torch.empty
@@ -60,6 +60,8 @@ class FusedLinear:
             elif self.in_heads is not None:
                 heads, real, pad = self.in_heads
                 out[join_name(name, self.suffix)] = Param(w.view(size, heads, pad)[:, :, :real], shape=(size, heads * real))
+                if b is not None:
+                    out[join_name(name, self.bias_suffix)] = Param(b)
             else:
                 out[join_name(name, self.suffix)] = Param(w)
                 if b is not None:

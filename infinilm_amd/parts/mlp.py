@@ -19,10 +19,11 @@ from .registry import register_feed_forward
 class SwiGLU(FeedForward):
     records_mixed_steps = True
 
-    def __init__(self, hidden_size: int, intermediate_size: int, bias: bool, ctx: BuildContext):
-        self.gate_up = FusedLinear(hidden_size, [intermediate_size, intermediate_size], ["gate_proj", "up_proj"],
-                                   bias, ctx)
-        self.down = Linear(intermediate_size, hidden_size, "down_proj", bias, ctx)
+    def __init__(self, hidden_size: int, intermediate_size: int, bias: bool, ctx: BuildContext,
+                 names=("gate_proj", "up_proj", "down_proj"), suffix: str = "weight"):
+        self.gate_up = FusedLinear(hidden_size, [intermediate_size, intermediate_size], [names[0], names[1]],
+                                   bias, ctx, suffix=suffix)
+        self.down = Linear(intermediate_size, hidden_size, names[2], bias, ctx, suffix=suffix)
 
     def named_parameters(self) -> Dict[str, Param]:
         out = dict(self.gate_up.named_parameters())

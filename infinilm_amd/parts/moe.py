@@ -80,3 +80,67 @@ class RoutedExperts(FeedForward):
             shared = self.shared_down.forward(kernels.glu_clamp(self.shared_gate_up.forward(x), self.shared_limit, self.alpha))
             gate = logits[:, self.E:]
         return kernels.moe_combine(pair_out, plan, shared, gate)
+
+
+@register_feed_forward("routed_activation_experts")
+class RoutedActivationExperts(FeedForward):
+    """Experts without a gate, weighed on their way out:
+
+      z = W_router h (float32)      s = softmax(z) over all experts (`router` = "softmax") or sigmoid(z) ("sigmoid")
+      y = sum over the `top` experts e with the largest s of  weight_scale * s_e * W_down,e act(W_up,e h)   (not renormalised)
+        + W_down,shared act(W_up,shared h)                                                           (if `shared_ff`)
+
+    `activation`: "relu2" (the square of relu) for the experts (the kernels' epilogue) and any of the kernels' activations
+    for the shared expert.  The experts' matrices lie stacked ([experts, ff, hidden], [experts, hidden, ff]); a checkpoint's
+    `e<j>.up`, `e<j>.down` are views into them.  Routing, ordering and the experts' products run on the device alone, as for
+    `routed_experts`; a pair's weight multiplies its expert's result in float32 when the token's results are summed."""
+    records_mixed_steps = True
+    trace: Optional[list] = None     # as `RoutedExperts.trace`
+
+    def __init__(self, hidden_size: int, experts: int, top: int, expert_ff: int, ctx: BuildContext, router: str = "softmax",
+                 weight_scale: float = 1.0, activation: str = "relu2", shared_ff: int = 0,
+                 names=("router", "e{}", "up", "down", "shared")):
+        self.W, self.E, self.top, self.ff = int(hidden_size), int(experts), int(top), int(expert_ff)
+        if not 1 <= self.top <= self.E:
+            raise ValueError(f"{self.top} of {self.E} experts a token")
+        if router not in ("softmax", "sigmoid"):
+            raise ValueError(f"unknown router {router!r} (softmax, sigmoid)")
+        if activation != "relu2":
+            raise ValueError(f"the experts' products take relu2 as their activation, got {activation!r}")
+        self.softmax, self.weight_scale, self.activation = router == "softmax", float(weight_scale), activation
+        self.shared_ff = int(shared_ff or 0)
+        self.names = tuple(names)
+        rn, en, un, dn, sn = self.names
+        self.dtype = ctx.dtype
+        self.router = Linear(self.W, self.E, rn, False, ctx, suffix="")
+        self.w_up = torch.empty((self.E, self.ff, self.W), dtype=ctx.dtype, device=ctx.device)
+        self.w_down = torch.empty((self.E, self.W, self.ff), dtype=ctx.dtype, device=ctx.device)
+        self.shared_up = self.shared_down = None
+        if self.shared_ff:
+            self.shared_up = Linear(self.W, self.shared_ff, f"{sn}.{un}", False, ctx, suffix="")
+            self.shared_down = Linear(self.shared_ff, self.W, f"{sn}.{dn}", False, ctx, suffix="")
+
+    def named_parameters(self) -> Dict[str, Param]:
+        rn, en, un, dn, sn = self.names
+        out = dict(self.router.named_parameters())
+        for e in range(self.E):
+            pre = en.format(e)
+            out[f"{pre}.{un}"] = Param(self.w_up[e])
+            out[f"{pre}.{dn}"] = Param(self.w_down[e])
+        if self.shared_ff:
+            out.update(self.shared_up.named_parameters())
+            out.update(self.shared_down.named_parameters())
+        return out
+
+    def forward(self, x, batch) -> torch.Tensor:
+        logits = kernels.gemm(x, self.router.weight, None, 1.0, torch.float32)          # [T, experts]
+        plan = kernels.moe_route(logits, self.E, self.top, softmax=self.softmax, weight_scale=self.weight_scale,
+                                 big_tiles_ok=x.dtype == torch.bfloat16 and self.W % 8 == 0 and self.ff % 8 == 0 and x.stride(0) % 8 == 0)
+        if RoutedActivationExperts.trace is not None:
+            RoutedActivationExperts.trace.append(plan.ids.clone())
+        act = kernels.moe_gemm(x, self.w_up, plan, False, gather=True, act=self.activation)   # [pairs, ff], ordered by expert
+        pair_out = kernels.moe_gemm(act, self.w_down, plan, False)                            # [pairs, hidden]
+        shared = None
+        if self.shared_ff:
+            shared = self.shared_down.forward(kernels.activation(self.shared_up.forward(x), self.activation))
+        return kernels.moe_combine(pair_out, plan, shared, None, weighted=True)

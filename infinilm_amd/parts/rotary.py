@@ -198,12 +198,18 @@ class NormedPairRotary(PositionEncoding):
     head_dim = 0    # any size the mixer runs: the entries beyond `dim` / `value_dim` are zeros
 
     def __init__(self, dim: int, value_dim: int, rotary_dim: int, theta: float, eps: float, ctx: BuildContext,
-                 qk_norm: bool = True, v_norm: bool = False, names=("q_norm", "k_norm")):
+                 qk_norm: bool = True, v_norm: bool = False, names=("q_norm", "k_norm"), frequencies=None):
         self.dim, self.value_dim, self.rotary_dim = int(dim), int(value_dim), int(rotary_dim)
         if self.rotary_dim % 2 or not 0 <= self.rotary_dim <= self.dim:
             raise ValueError(f"rotary_dim {rotary_dim} must be even and at most the head size {dim}")
         self.eps, self.v_norm, self.names = float(eps), bool(v_norm), tuple(names)
-        self.freq = pair_frequencies(self.rotary_dim, theta, ctx.device)
+        # `frequencies`: the rotary_dim / 2 turning rates themselves (a design that scales them), in place of theta^(-2i/dims)
+        if frequencies is not None and self.rotary_dim:
+            if len(frequencies) != self.rotary_dim // 2:
+                raise ValueError(f"{len(frequencies)} frequencies for {self.rotary_dim // 2} pairs")
+            self.freq = torch.tensor(list(frequencies), dtype=torch.float64).to(torch.float32).to(ctx.device)
+        else:
+            self.freq = pair_frequencies(self.rotary_dim, theta, ctx.device)
         self.q_weight = torch.empty((self.dim,), dtype=ctx.dtype, device=ctx.device) if qk_norm else None
         self.k_weight = torch.empty((self.dim,), dtype=ctx.dtype, device=ctx.device) if qk_norm else None
 
