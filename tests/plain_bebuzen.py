@@ -17,6 +17,13 @@ from typing import Dict, List, Optional
 import torch
 
 F64 = torch.float64
+_ROUND = None      # a dtype: `forward(..., round_to=)` rounds what an engine in that dtype rounds (see `_r`)
+
+
+def _r(x: torch.Tensor) -> torch.Tensor:
+    """x as it is, or rounded to the dtype a run of `forward` asked for: the rows a projection reads, its result, the normed
+    and turned queries and keys, an attention's result.  What the design computes in 32-bit is never rounded."""
+    return x if _ROUND is None else x.to(_ROUND).to(F64)
 
 
 def rms(x: torch.Tensor, eps: float, w: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -115,25 +122,25 @@ def differential_keys_values(W: Dict[str, torch.Tensor], p: str, mx: dict, h: to
     """The keys (after convolution, norm and rotation) [T, G, 2, dim] and values (after convolution) [T, G, vdim]."""
     G, dim, vdim = int(mx["kv_heads"]), int(mx["dim"]), int(mx["vdim"])
     T = h.shape[0]
-    k = h @ W[p + "k"].T + W[p + "k.b"]
-    v = h @ W[p + "v"].T + W[p + "v.b"]
+    k = _r(h @ W[p + "k"].T + W[p + "k.b"])
+    v = _r(h @ W[p + "v"].T + W[p + "v.b"])
     if mx.get("conv"):
         k = short_conv(k, W[p + "k.conv"])
         v = short_conv(v, W[p + "v.conv"])
     k = rms(k.view(T, G * 2, dim), eps, W[p + "k.norm"])
-    k = rotate(k, pos, mx.get("rot"), "half")
-    return k.view(T, G, 2, dim), v.view(T, G, vdim)
+    k = _r(rotate(k, pos, mx.get("rot"), "half"))
+    return k.view(T, G, 2, dim), _r(v).view(T, G, vdim)
 
 
 def differential_attention(W, p: str, mx: dict, h, pos, eps: float, kv=None):
     """Returns (output [T, width], (k, v)); `kv`: another layer's keys and values to read instead of one's own."""
     H, G, dim, vdim = int(mx["heads"]), int(mx["kv_heads"]), int(mx["dim"]), int(mx["vdim"])
     T = h.shape[0]
-    q = h @ W[p + "q"].T + W[p + "q.b"]
+    q = _r(h @ W[p + "q"].T + W[p + "q.b"])
     if mx.get("conv"):
         q = short_conv(q, W[p + "q.conv"])
     q = rms(q.view(T, H * 2, dim), eps, W[p + "q.norm"])
-    q = rotate(q, pos, mx.get("rot"), "half").view(T, H, 2, dim)
+    q = _r(rotate(q, pos, mx.get("rot"), "half")).view(T, H, 2, dim)
     if kv is None:
         kv = differential_keys_values(W, p, mx, h, pos, eps)
     k, v = kv
@@ -143,55 +150,59 @@ def differential_attention(W, p: str, mx: dict, h, pos, eps: float, kv=None):
     a2 = softmax_attention(q[:, :, 1], k[:, :, 1], v, float(mx["scale"]), mask, False)
     diff = float(mx["diff"])
     lam = torch.exp((W[p + "lq1"] * W[p + "lk1"]).sum()) - torch.exp((W[p + "lq2"] * W[p + "lk2"]).sum()) + diff
-    o = rms(a1 - lam * a2, eps) * (1.0 - diff)
-    return o.reshape(T, H * vdim) @ W[p + "o"].T, kv
+    o = _r(rms(a1 - lam * a2, eps) * (1.0 - diff))
+    return _r(o.reshape(T, H * vdim) @ W[p + "o"].T), kv
 
 
 def sink_window_attention(W, p: str, mx: dict, h, pos, eps: float):
     H, G, dim, vdim = int(mx["heads"]), int(mx["kv_heads"]), int(mx["dim"]), int(mx["vdim"])
     T = h.shape[0]
-    q = (h @ W[p + "q"].T + W[p + "q.b"]).view(T, H, dim)
-    k = (h @ W[p + "k"].T + W[p + "k.b"]).view(T, G, dim)
-    v = (h @ W[p + "v"].T + W[p + "v.b"]).view(T, G, vdim)
-    q = rotate(rms(q, eps, W[p + "q.norm"]), pos, mx.get("rot"), "pairs")
-    k = rotate(rms(k, eps, W[p + "k.norm"]), pos, mx.get("rot"), "pairs")
+    q = _r(h @ W[p + "q"].T + W[p + "q.b"]).view(T, H, dim)
+    k = _r(h @ W[p + "k"].T + W[p + "k.b"]).view(T, G, dim)
+    v = _r(h @ W[p + "v"].T + W[p + "v.b"]).view(T, G, vdim)
+    q = _r(rotate(rms(q, eps, W[p + "q.norm"]), pos, mx.get("rot"), "pairs"))
+    k = _r(rotate(rms(k, eps, W[p + "k.norm"]), pos, mx.get("rot"), "pairs"))
     mk = mx.get("mask")
     mask = visible(T, mk["size"] if mk else None, int(mk.get("keep_first", 0)) if mk else 0)
-    o = softmax_attention(q, k, v, float(mx["scale"]), mask, True)
-    return o.reshape(T, H * vdim) @ W[p + "o"].T + W[p + "o.b"]
+    o = _r(softmax_attention(q, k, v, float(mx["scale"]), mask, True))
+    return _r(o.reshape(T, H * vdim) @ W[p + "o"].T + W[p + "o.b"])
 
 
 def selective_scan(W, p: str, mx: dict, h):
     inner, state, dt_rank = int(mx["inner"]), int(mx["state"]), int(mx["dt_rank"])
     T = h.shape[0]
-    xz = h @ W[p + "in"].T
+    xz = _r(h @ W[p + "in"].T)
     x, z = xz[:, :inner], xz[:, inner:]
     x = silu(short_conv(x, W[p + "conv"], W[p + "conv.b"]))
-    r = x @ W[p + "x"].T
+    r = _r(_r(x) @ W[p + "x"].T)
     dt, B, C = r[:, :dt_rank], r[:, dt_rank:dt_rank + state], r[:, dt_rank + state:]
-    dt = torch.nn.functional.softplus(dt @ W[p + "dt"].T + W[p + "dt.b"])
+    dt = torch.nn.functional.softplus(_r(dt @ W[p + "dt"].T) + W[p + "dt.b"])
     A = -torch.exp(W[p + "A_log"])
     S = torch.zeros((inner, state), dtype=h.dtype)
     ys = []
     for t in range(T):
         S = torch.exp(dt[t][:, None] * A) * S + (dt[t] * x[t])[:, None] * B[t][None, :]
         ys.append(S @ C[t] + W[p + "D"] * x[t])
-    y = torch.stack(ys) * silu(z)
-    return y @ W[p + "o"].T
+    y = _r(torch.stack(ys) * silu(z))
+    return _r(y @ W[p + "o"].T)
 
 
 def relu2_mlp(W, p: str, h):
-    return torch.relu(h @ W[p + "up"].T) ** 2 @ W[p + "down"].T
+    return _r(_r(torch.relu(_r(h @ W[p + "up"].T)) ** 2) @ W[p + "down"].T)
 
 
-def feed_forward(W, p: str, ml: dict, h, forced: Optional[torch.Tensor] = None):
-    """`forced` [T, top]: expert choices to use instead of the router's own (the weights still come from the scores)."""
+def feed_forward(W, p: str, ml: dict, h, forced: Optional[torch.Tensor] = None, chosen: Optional[list] = None):
+    """`forced` [T, top]: expert choices to use instead of the router's own (the weights still come from the scores);
+    `chosen`: a list that receives (the router's own choices [T, top], the scores [T, experts])."""
     if ml["kind"] == "dense":
-        return (silu(h @ W[p + "gate"].T) * (h @ W[p + "up"].T)) @ W[p + "down"].T
+        return _r(_r(silu(_r(h @ W[p + "gate"].T)) * _r(h @ W[p + "up"].T)) @ W[p + "down"].T)
     r = ml["router"]
     E, top = int(r["experts"]), int(r["top"])
     s = torch.softmax(h @ W[p + "router"].T, -1)
-    idx = forced if forced is not None else torch.topk(s, top, dim=-1).indices
+    own = torch.topk(s, top, dim=-1).indices
+    if chosen is not None:
+        chosen.append((own, s))
+    idx = forced if forced is not None else own
     out = torch.zeros_like(h)
     for e in range(E):
         rows = (idx == e).any(-1).nonzero().flatten()
@@ -202,8 +213,21 @@ def feed_forward(W, p: str, ml: dict, h, forced: Optional[torch.Tensor] = None):
     return out
 
 
-def forward(cfg: dict, W: Dict[str, torch.Tensor], tokens: List[int], return_layers: bool = False, forced: Optional[dict] = None):
-    """Logits [T, vocab] of one sequence from its start (and the stream after every layer)."""
+def forward(cfg: dict, W: Dict[str, torch.Tensor], tokens: List[int], return_layers: bool = False, forced: Optional[dict] = None,
+            chosen: Optional[dict] = None, round_to: Optional[torch.dtype] = None):
+    """Logits [T, vocab] of one sequence from its start (and the stream after every layer).  `forced` {layer: [T, top]}: expert
+    choices to use; `chosen`: a dict that receives {layer: (the router's own choices, the scores)}; `round_to`: a dtype to which
+    the rows a projection reads and what it gives are rounded, as an engine in that dtype does (the stream, norms, scores,
+    states and routers stay exact)."""
+    global _ROUND
+    _ROUND = round_to
+    try:
+        return _forward(cfg, W, tokens, return_layers, forced, chosen)
+    finally:
+        _ROUND = None
+
+
+def _forward(cfg, W, tokens, return_layers, forced, chosen):
     W = {k: v.to(F64) for k, v in W.items()}
     eps, m = float(cfg["norm"]["eps"]), float(cfg.get("residual_mult", 1.0))
     x = W["embed"][torch.tensor(tokens)]
@@ -213,20 +237,23 @@ def forward(cfg: dict, W: Dict[str, torch.Tensor], tokens: List[int], return_lay
         p, mx = f"l{i}.mix.", ly["mixer"]
         if ly["type"] == "attention":
             src = mx.get("kv_from")
-            y, kv = differential_attention(W, p, mx, x, pos, eps, kvs[src] if src is not None else None)
+            y, kv = differential_attention(W, p, mx, _r(x), pos, eps, kvs[src] if src is not None else None)
             kvs[i] = kv
         elif ly["type"] == "attention_2":
-            y = sink_window_attention(W, p, mx, x, pos, eps)
+            y = sink_window_attention(W, p, mx, _r(x), pos, eps)
         elif ly["type"] == "mamba1":
-            y = selective_scan(W, p, mx, x)
+            y = selective_scan(W, p, mx, _r(x))
         else:
             raise ValueError(ly["type"])
         x = x + m * rms(y, eps, W[f"l{i}.norm1"])
         if ly.get("mlp"):
-            y = feed_forward(W, f"l{i}.mlp.", ly["mlp"], x, None if forced is None else forced.get(i))
+            got = [] if chosen is not None else None
+            y = feed_forward(W, f"l{i}.mlp.", ly["mlp"], _r(x), None if forced is None else forced.get(i), got)
+            if got:
+                chosen[i] = got[0]
             x = x + m * rms(y, eps, W[f"l{i}.norm2"])
         layers.append(x.clone())
-    logits = rms(x, eps, W["final.norm"]) @ W["head"].T
+    logits = _r(rms(x, eps, W["final.norm"])) @ W["head"].T
     return (logits, torch.stack(layers)) if return_layers else logits
 
 
@@ -282,4 +309,85 @@ def tensor_shapes(cfg: dict) -> Dict[str, tuple]:
                     out[q + "shared.down"] = (Wd, sf)
     out["final.norm"] = (Wd,)
     out["head"] = (int(cfg["vocab"]), Wd)
+    return out
+
+
+# ---- configurations and weights for tests --------------------------------------------------------------------------------
+def _scaling():
+    return {"factor": 4.0, "low": 1.0, "high": 3.0, "original": 64}
+
+
+def config_a():
+    moe = {"kind": "moe", "router": {"experts": 4, "top": 2, "scale": 1.5}, "expert": {"ff": 24}, "shared": {"ff": 16}}
+    return {"architecture": "Bebuzen", "vocab": 97, "width": 64, "norm": {"eps": 1e-5}, "residual_mult": 0.5, "layers": [
+        {"type": "attention_2", "mixer": {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 24, "scale": 0.3, "rot": {"base": 100.0, "dims": 8},
+                                          "mask": {"size": 20, "keep_first": 3}}, "mlp": {"kind": "dense", "ff": 48}},
+        {"type": "attention", "mixer": {"heads": 2, "kv_heads": 1, "dim": 8, "vdim": 12, "scale": 0.4, "diff": 0.3, "conv": 2,
+                                        "rot": {"base": 50.0, "dims": 8, "scaling": _scaling()}, "mask": {"size": 33}}, "mlp": moe},
+        {"type": "mamba1", "mixer": {"inner": 48, "state": 5, "dt_rank": 3, "conv": 4}, "mlp": None},
+        {"type": "attention", "mixer": {"heads": 2, "kv_heads": 1, "dim": 8, "vdim": 12, "scale": 0.4, "diff": 0.3, "conv": 2,
+                                        "rot": {"base": 50.0, "dims": 8, "scaling": _scaling()}, "mask": {"size": 50}, "kv_from": 1}, "mlp": moe}]}
+
+
+def config_b():
+    moe = {"kind": "moe", "router": {"experts": 3, "top": 1}, "expert": {"ff": 20}}
+    return {"architecture": "Bebuzen", "vocab": 130, "width": 96, "norm": {"eps": 1e-6}, "layers": [
+        {"type": "mamba1", "mixer": {"inner": 160, "state": 20, "dt_rank": 7, "conv": 2}, "mlp": {"kind": "dense", "ff": 72}},
+        {"type": "attention", "mixer": {"heads": 6, "kv_heads": 6, "dim": 12, "vdim": 8, "scale": 0.25, "diff": 0.7, "conv": 4,
+                                        "rot": {"base": 1000.0, "dims": 4}}, "mlp": moe},
+        {"type": "attention_2", "mixer": {"heads": 3, "kv_heads": 1, "dim": 32, "vdim": 32, "scale": 0.2, "mask": {"size": 64}}, "mlp": moe},
+        {"type": "attention_2", "mixer": {"heads": 2, "kv_heads": 2, "dim": 20, "vdim": 36, "scale": 0.2, "rot": {"base": 10000.0, "dims": 20}},
+         "mlp": None},
+        {"type": "attention", "mixer": {"heads": 6, "kv_heads": 6, "dim": 12, "vdim": 8, "scale": 0.25, "diff": 0.7, "conv": 4,
+                                        "rot": {"base": 1000.0, "dims": 4}, "kv_from": 1}, "mlp": {"kind": "dense", "ff": 40}}]}
+
+
+def config_c():
+    """Sizes the matrix-core kernels take."""
+    moe = {"kind": "moe", "router": {"experts": 8, "top": 3, "scale": 2.0}, "expert": {"ff": 64}, "shared": {"ff": 64}}
+    rot = {"base": 5000.0, "dims": 32, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 128}}
+    return {"architecture": "Bebuzen", "vocab": 200, "width": 128, "norm": {"eps": 1e-5}, "residual_mult": 0.8, "layers": [
+        {"type": "attention", "mixer": {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 64, "scale": 0.18, "diff": 0.5, "conv": 3,
+                                        "rot": rot, "mask": {"size": 70}}, "mlp": {"kind": "dense", "ff": 256}},
+        {"type": "attention_2", "mixer": {"heads": 4, "kv_heads": 2, "dim": 64, "vdim": 64, "scale": 0.125, "rot": {"base": 10000.0, "dims": 32},
+                                          "mask": {"size": 40, "keep_first": 5}}, "mlp": moe},
+        {"type": "attention", "mixer": {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 64, "scale": 0.18, "diff": 0.5, "conv": 3,
+                                        "rot": rot, "mask": {"size": 70}, "kv_from": 0}, "mlp": moe},
+        {"type": "mamba1", "mixer": {"inner": 256, "state": 16, "dt_rank": 8, "conv": 4}, "mlp": {"kind": "dense", "ff": 128}}]}
+
+
+CONFIGS = {"A": config_a, "B": config_b, "C": config_c}
+
+
+def random_weights(cfg: dict, seed: int) -> Dict[str, torch.Tensor]:
+    """float32 tensors of a size that keeps every mechanism at work: norms near one, decays spread over (0, 1), routers sharp
+    enough that the chosen experts seldom hang on a rounding."""
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, shape in tensor_shapes(cfg).items():
+        leaf = name.split(".")[-1]
+        r = torch.randn(shape, generator=g)
+        if leaf in ("norm1", "norm2", "norm") or name == "final.norm":
+            t = 1.0 + 0.2 * r
+        elif name.endswith("A_log"):
+            t = torch.log(0.3 + 3.0 * torch.rand(shape, generator=g))
+        elif name.endswith("dt.b"):
+            t = -2.5 + 0.8 * r
+        elif leaf == "D":
+            t = 1.0 + 0.3 * r
+        elif leaf in ("lq1", "lk1", "lq2", "lk2"):
+            t = 0.3 * r
+        elif leaf == "b":
+            t = 0.2 * r
+        elif leaf == "conv":
+            t = 0.6 * r
+        elif leaf == "router":
+            t = 3.0 * r / math.sqrt(shape[1])
+        elif name == "embed":
+            t = r
+        elif len(shape) == 2:
+            t = r * (1.3 / math.sqrt(shape[1]))
+        else:
+            t = r
+        out[name] = t
     return out
