@@ -6,6 +6,10 @@
 //       dim entries is RMS-normed with a weight shared by all units (or none) and its first rd entries are turned in the
 //       pairs (i, i + rd/2) by the angle pos * freq[i]; q goes to dense rows [T, H maps dim], k to the paged cache with a
 //       key/value head's maps side by side ([pages, G, page, d], entry m dim + e), v to the transposed value cache.
+//       `spread`: the queries go out as rows of G x d entries a unit instead (zeros but for the unit's own group and map),
+//       which is how the matrix-core attention that asks all groups at once takes them.
+//   ilm_maps_combine             from float rows [T, H 2, d] of the two maps' results: o = a_0 - lambda a_1, its root mean
+//       square over the head's vdim entries, the scale (the end of ilm_attn_maps, for results that another kernel made).
 //   ilm_attn_maps                per query head h (key/value head h / (H/G)) and map m a softmax attention of its own over
 //       the keys the token sees (j <= i and (i - j < window or j < keep_first); window 0: all), scores scale q_hm . k_gm,
 //       optionally one more term exp(sink) in every denominator; the maps' results a_m share the values.  One map: o = a_0.
@@ -22,7 +26,7 @@ __global__ void __launch_bounds__(256)
 maps_norm_rope_kvwrite_kernel(T* __restrict__ q_out, const TS* __restrict__ src, int stride, int q_off, int k_off, int v_off,
                               const int* __restrict__ pos, const float* __restrict__ freq, const TW* __restrict__ wq,
                               const TW* __restrict__ wk, T* __restrict__ kc, T* __restrict__ vc, const int* __restrict__ slots,
-                              int H, int G, int maps, int dim, int vdim, int d, int rd, float eps, int page) {
+                              int H, int G, int maps, int dim, int vdim, int d, int rd, float eps, int page, int spread) {
     extern __shared__ float smem[];
     const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int nq = H * maps, nk = k_off >= 0 ? G * maps : 0, nv = k_off >= 0 ? G : 0;
@@ -49,21 +53,30 @@ maps_norm_rope_kvwrite_kernel(T* __restrict__ q_out, const TS* __restrict__ src,
         for (int e = lane; e < n; e += 64) x[e] = x[e] * rstd * to_f32(w[e]);
     }
     __syncthreads();
-    float turned_u = 0.f, turned_v = 0.f;
     const int half = rd / 2;
     if (active && (is_q || is_k) && rd > 0) {
         const float ps = (float)pos[t];
-        for (int i = lane; i < half; i += 64) {      // (half <= 64 a round in all usual sizes; the loop keeps one pair a lane in flight)
+        for (int i = lane; i < half; i += 64) {      // (a pair a lane and round; no pair is touched by two lanes)
             float sn, cs;
             sincosf(ps * freq[i], &sn, &cs);
-            turned_u = x[i] * cs - x[i + half] * sn;
-            turned_v = x[i + half] * cs + x[i] * sn;
-            x[i] = turned_u;
-            x[i + half] = turned_v;
+            const float u = x[i], v = x[i + half];
+            x[i] = u * cs - v * sn;
+            x[i + half] = v * cs + u * sn;
         }
     }
     __syncthreads();
     if (!active) return;
+    if (is_q && spread) {
+        // for the matrix-core kernel that asks every key/value group with one query of G x d entries: unit (h, m) is zeros
+        // but for its own group's entries m dim .. (m + 1) dim - 1, so that its score is q_hm . k_gm and nothing else
+        const int g = (unit / maps) / (H / G), m = unit % maps;
+        T* dst = q_out + ((size_t)t * nq + unit) * G * d;
+        for (int e = lane; e < G * d; e += 64) {
+            const int c = e / d, i = e % d - m * dim;
+            dst[e] = from_f32<T>((c == g && i >= 0 && i < dim) ? x[i] : 0.f);
+        }
+        return;
+    }
     if (is_q) {
         T* dst = q_out + (size_t)t * nq * dim + (size_t)unit * dim;
         for (int e = lane; e < dim; e += 64) dst[e] = from_f32<T>(x[e]);
@@ -86,7 +99,8 @@ maps_norm_rope_kvwrite_kernel(T* __restrict__ q_out, const TS* __restrict__ src,
 extern "C" int ilm_maps_norm_rope_kvwrite(void* q_out, const void* src, int stride, int q_off, int k_off, int v_off, const void* pos,
                                           const void* freq, const void* wq, const void* wk, void* kc, void* vc, const void* slots,
                                           int T_, int H, int G, int maps, int dim, int vdim, int d, int rd, float eps, int page,
-                                          int src_dt, int dtype, int w_dt, hipStream_t stream) {
+                                          int src_dt, int dtype, int w_dt, int spread, hipStream_t stream) {
+    ILM_REQUIRE(!spread || (H % G == 0 && maps * dim <= d), "maps_norm_rope_kvwrite: queries spread over %d groups of %d", G, d);
     ILM_REQUIRE(T_ > 0 && H > 0 && G > 0 && maps > 0 && dim > 0 && vdim > 0 && page > 0, "maps_norm_rope_kvwrite: bad sizes");
     ILM_REQUIRE(k_off < 0 || (maps * dim <= d && vdim <= d), "maps_norm_rope_kvwrite: %d maps of %d / values of %d in cache heads of %d", maps,
                 dim, vdim, d);
@@ -99,7 +113,7 @@ extern "C" int ilm_maps_norm_rope_kvwrite(void* q_out, const void* src, int stri
 #define MP_LAUNCH(TS__, T__, TW__)                                                                                           \
     maps_norm_rope_kvwrite_kernel<TS__, T__, TW__><<<grid, 256, shm, stream>>>(                                              \
         (T__*)q_out, (const TS__*)src, stride, q_off, k_off, v_off, (const int*)pos, (const float*)freq, (const TW__*)wq,    \
-        (const TW__*)wk, (T__*)kc, (T__*)vc, (const int*)slots, H, G, maps, dim, vdim, d, rd, eps, page)
+        (const TW__*)wk, (T__*)kc, (T__*)vc, (const int*)slots, H, G, maps, dim, vdim, d, rd, eps, page, spread)
     if (src_dt == ILM_DTYPE_F32 && dtype == ILM_DTYPE_F32 && w_dt == ILM_DTYPE_F32) MP_LAUNCH(float, float, float);
     else if (src_dt == ILM_DTYPE_F32 && dtype == ILM_DTYPE_BF16 && w_dt == ILM_DTYPE_BF16) MP_LAUNCH(float, bf16, bf16);
     else if (src_dt == ILM_DTYPE_F32 && dtype == ILM_DTYPE_BF16 && w_dt == ILM_DTYPE_F32) MP_LAUNCH(float, bf16, float);
@@ -287,5 +301,56 @@ extern "C" int ilm_attn_maps(void* out, const void* q, const void* kc, const voi
     else ILM_REQUIRE(false, "attn_maps: dtypes %d / %d", dtype, w_dt);
 #undef AM_LAUNCH
     ILM_LAUNCH_CHECK("attn_maps");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// One wave a (token, head): o = a_0 - lambda a_1 over vdim entries of float rows [T, H 2, d], normed and scaled.
+// ------------------------------------------------------------------------------------------
+template <typename T, typename TW>
+__global__ void __launch_bounds__(256)
+maps_combine_kernel(T* __restrict__ out, const float* __restrict__ a, int T_, int H, int vdim, int d, int out_stride,
+                    const TW* __restrict__ lq1, const TW* __restrict__ lk1, const TW* __restrict__ lq2, const TW* __restrict__ lk2,
+                    float diff, float norm_eps, float out_scale, int dim) {
+    const int lane = threadIdx.x & 63;
+    const long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (item >= (long)T_ * H) return;
+    const int t = (int)(item / H), h = (int)(item % H);
+    float x = 0.f, y = 0.f;
+    for (int e = lane; e < dim; e += 64) {
+        x = fmaf(to_f32(lq1[e]), to_f32(lk1[e]), x);
+        y = fmaf(to_f32(lq2[e]), to_f32(lk2[e]), y);
+    }
+    const float lambda = expf(wave_sum(x)) - expf(wave_sum(y)) + diff;
+    const float* a0 = a + ((size_t)t * H + h) * 2 * d;
+    const float* a1 = a0 + d;
+    float ss = 0.f;
+    for (int e = lane; e < vdim; e += 64) {
+        const float o = a0[e] - lambda * a1[e];
+        ss = fmaf(o, o, ss);
+    }
+    ss = wave_sum(ss);
+    const float f = norm_eps >= 0.f ? out_scale / sqrtf(ss / (float)vdim + norm_eps) : out_scale;
+    T* orow = out + (size_t)t * out_stride + (size_t)h * vdim;
+    for (int e = lane; e < vdim; e += 64) orow[e] = from_f32<T>((a0[e] - lambda * a1[e]) * f);
+}
+
+extern "C" int ilm_maps_combine(void* out, const void* a, int T_, int H, int vdim, int d, int out_stride, const void* lq1, const void* lk1,
+                                const void* lq2, const void* lk2, float diff, float norm_eps, float out_scale, int dim, int w_dt,
+                                hipStream_t stream) {
+    ILM_REQUIRE(T_ > 0 && H > 0 && vdim > 0 && vdim <= d && dim > 0 && out_stride >= H * vdim, "maps_combine: bad sizes");
+    ILM_REQUIRE(lq1 && lk1 && lq2 && lk2, "maps_combine: the four vectors of the maps' weight are needed");
+    const unsigned blocks = (unsigned)(((long)T_ * H + 3) / 4);
+    if (w_dt == ILM_DTYPE_BF16)
+        maps_combine_kernel<bf16, bf16><<<blocks, 256, 0, stream>>>((bf16*)out, (const float*)a, T_, H, vdim, d, out_stride, (const bf16*)lq1,
+                                                                   (const bf16*)lk1, (const bf16*)lq2, (const bf16*)lk2, diff, norm_eps,
+                                                                   out_scale, dim);
+    else if (w_dt == ILM_DTYPE_F32)
+        maps_combine_kernel<bf16, float><<<blocks, 256, 0, stream>>>((bf16*)out, (const float*)a, T_, H, vdim, d, out_stride, (const float*)lq1,
+                                                                    (const float*)lk1, (const float*)lq2, (const float*)lk2, diff, norm_eps,
+                                                                    out_scale, dim);
+    else
+        ILM_REQUIRE(false, "maps_combine: dtype %d", w_dt);
+    ILM_LAUNCH_CHECK("maps_combine");
     return 0;
 }

@@ -103,7 +103,8 @@ attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, co
                          const int* __restrict__ block_tables, const int* __restrict__ seg, const int* __restrict__ pos,
                          const int* __restrict__ tiles, int n_tiles, const int* __restrict__ singles,
                          const float* __restrict__ sink, int nh, int page, int max_blocks, int out_stride, float scale_log2e,
-                         int window, float* __restrict__ ws, int chunk_keys, const int* __restrict__ seg_offsets, int keep_first) {
+                         int window, float* __restrict__ ws, int chunk_keys, const int* __restrict__ seg_offsets, int keep_first,
+                         int out_f32) {
     constexpr int D = D32 * 32, KROW = D + 8, VROW = TK + 8, NS = TK / 16, NP = TK / 32;
     extern __shared__ __attribute__((aligned(16))) unsigned char hx_smem[];
     bf16* Ks = reinterpret_cast<bf16*>(hx_smem);                 // [NC][32][KROW]
@@ -305,7 +306,14 @@ attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, co
         }
         if (sink != nullptr) l += __builtin_amdgcn_exp2f(sink[head[i]] * 1.4426950408889634f - m_run[i]);
         const float inv = 1.0f / l;
-        if (tok_ok && lane_ok[i]) {
+        if (tok_ok && lane_ok[i] && out_f32) {       // (float rows for a caller that goes on in float: `out` then points to floats)
+            float* orow = reinterpret_cast<float*>(out) + (size_t)tok * out_stride + (size_t)head[i] * D;
+#pragma unroll
+            for (int b = 0; b < 2 * D32; ++b) {
+                const hx_f32x4 o = O[i][b];
+                *reinterpret_cast<float4*>(orow + b * 16 + g4 * 4) = make_float4(o[0] * inv, o[1] * inv, o[2] * inv, o[3] * inv);
+            }
+        } else if (tok_ok && lane_ok[i]) {
             bf16* orow = out + (size_t)tok * out_stride + (size_t)head[i] * D;
 #pragma unroll
             for (int b = 0; b < 2 * D32; ++b) {
@@ -319,7 +327,7 @@ attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, co
 // the chunks' partial results of a single token and head folded in order, the sink's term, the division
 __global__ void __launch_bounds__(128)
 attn_headmix_merge_kernel(bf16* __restrict__ out, const float* __restrict__ ws, const int* __restrict__ singles,
-                          const float* __restrict__ sink, int nh, int D, int nz, int out_stride) {
+                          const float* __restrict__ sink, int nh, int D, int nz, int out_stride, int out_f32) {
     const int item = blockIdx.x, h = blockIdx.y, e = threadIdx.x;
     const int t = singles != nullptr ? singles[item] : item;
     if (t < 0 || e >= D) return;
@@ -334,7 +342,8 @@ attn_headmix_merge_kernel(bf16* __restrict__ out, const float* __restrict__ ws, 
         M = Mn;
     }
     if (sink != nullptr) L += __builtin_amdgcn_exp2f(sink[h] * 1.4426950408889634f - M);
-    out[(size_t)t * out_stride + (size_t)h * D + e] = from_f32<bf16>(A / L);
+    if (out_f32) reinterpret_cast<float*>(out)[(size_t)t * out_stride + (size_t)h * D + e] = A / L;
+    else out[(size_t)t * out_stride + (size_t)h * D + e] = from_f32<bf16>(A / L);
 }
 
 extern "C" int ilm_attn_headmix_mfma_ok(int nh, int nkv, int d, int page) {
@@ -350,7 +359,7 @@ extern "C" int ilm_attn_headmix_mfma(void* out, const void* qx, const void* kc, 
                                      const void* seg, const void* pos, const void* tiles, int n_tiles, const void* singles,
                                      int n_singles, const void* sink, int nh, int nkv, int d, int page, int max_blocks,
                                      int out_stride, float scale, int window, void* ws, int nz, int chunk_keys,
-                                     const void* seg_offsets, int keep_first, hipStream_t stream) {
+                                     const void* seg_offsets, int keep_first, int out_f32, hipStream_t stream) {
     ILM_REQUIRE(keep_first >= 0, "attn_headmix_mfma: %d kept first tokens", keep_first);
     // single tokens whose heads come in groups of a multiple of 16: heads as the products' columns
     // (a block of 16 columns must lie in one key/value group: one group in all, or groups of a multiple of 16 heads)
@@ -361,6 +370,7 @@ extern "C" int ilm_attn_headmix_mfma(void* out, const void* qx, const void* kc, 
     if (ws == nullptr) { nz = 1; chunk_keys = 0; }
     ILM_REQUIRE(n_tiles >= 0 && n_singles >= 0 && n_tiles + n_singles > 0 && max_blocks > 0, "attn_headmix_mfma: bad sizes");
     ILM_REQUIRE(ilm_attn_headmix_mfma_ok(nh, nkv, d, page), "attn_headmix_mfma: %d heads in %d groups of %d, pages of %d", nh, nkv, d, page);
+    ILM_REQUIRE(!out_f32 || ((uintptr_t)out & 15) == 0, "attention_headmix_mfma: float rows must be 16-byte aligned");
     ILM_REQUIRE(out_stride % 4 == 0 && ((uintptr_t)out & 7) == 0 && ((uintptr_t)qx & 15) == 0 && ((uintptr_t)kc & 15) == 0 &&
                 ((uintptr_t)vc & 15) == 0, "attn_headmix_mfma: rows must be 16-byte / 8-byte aligned");
     const float scale_log2e = scale * 1.4426950408889634f;
@@ -379,7 +389,7 @@ extern "C" int ilm_attn_headmix_mfma(void* out, const void* qx, const void* kc, 
                                          (const int*)block_tables, (const int*)seg, (const int*)pos, (const int*)tiles,    \
                                          n_tiles, (const int*)singles, (const float*)sink, nh, page, max_blocks,           \
                                          out_stride, scale_log2e, window, (float*)ws, chunk_keys,                          \
-                                         (const int*)seg_offsets, keep_first);                                             \
+                                         (const int*)seg_offsets, keep_first, out_f32);                                    \
     }
 #define HX_BY_NC(D32_)                                                      \
     switch (nkv) {                                                          \
@@ -399,7 +409,7 @@ extern "C" int ilm_attn_headmix_mfma(void* out, const void* qx, const void* kc, 
     ILM_LAUNCH_CHECK("attn_headmix_mfma");
     if (ws != nullptr) {
         attn_headmix_merge_kernel<<<dim3(n_singles, nh), 128, 0, stream>>>((bf16*)out, (const float*)ws, (const int*)singles,
-                                                                           (const float*)sink, nh, d, nz, out_stride);
+                                                                           (const float*)sink, nh, d, nz, out_stride, out_f32);
         ILM_LAUNCH_CHECK("attn_headmix_mfma (merge)");
     }
     return 0;

@@ -58,7 +58,7 @@ _SIGNATURES = {
     "ilm_qkv_norm_rope_kvwrite": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P],
     "ilm_attn_headmix": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
     "ilm_headmix_queries": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
-    "ilm_attn_headmix_mfma": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _I, _I, _P, _I, _P],
+    "ilm_attn_headmix_mfma": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _I, _I, _P, _I, _I, _P],
     "ilm_latent_prep": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _P],
     "ilm_embed_pos": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _P],
     "ilm_stream_update": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _F, _F, _I, _I, _I, _I, _I, _L, _I, _I, _P],
@@ -68,7 +68,8 @@ _SIGNATURES = {
     "ilm_moe_sort": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
     "ilm_moe_gemm": [_P, _I, _P, _I, _P, _I, _P, _P, _L, _I, _P, _P, _I, _I, _I, _I, _F, _F, _I, _I, _I, _I, _I, _P],
     "ilm_moe_combine": [_P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _P, _I, _P],
-    "ilm_maps_norm_rope_kvwrite": [_P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P],
+    "ilm_maps_norm_rope_kvwrite": [_P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _P],
+    "ilm_maps_combine": [_P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _F, _F, _F, _I, _I, _P],
     "ilm_attn_maps": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P, _P, _P, _P, _F, _F, _F,
                       _I, _I, _P],
     "ilm_selective_scan": [_P, _I, _P, _I, _P, _I, _P, _P, _P, _I, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],

@@ -1366,7 +1366,7 @@ def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                       window: int = 0, mix: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None,
                       tiles: Optional[torch.Tensor] = None, single_rows: Optional[torch.Tensor] = None,
                       max_total_len: Optional[int] = None, seg_offsets: Optional[torch.Tensor] = None,
-                      keep_first: int = 0) -> torch.Tensor:
+                      keep_first: int = 0, spread_queries: bool = False, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """Attention of every token over its request's cached keys (its last `window` positions, or all; with `keep_first` the
     sequence's first that many keys stay seen however far the window has moved) where the scaled
     scores of the heads are mixed before the softmax, s_h = sum_g mix[h, g] raw_g (`mix` float32 [nh, nh] or None),
@@ -1377,8 +1377,18 @@ def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     every token is served on its own); the matrix-core kernel (bfloat16, heads of 32 to 128 in steps of 32, 1, 2 or 4
     key/value groups, pages of a multiple of 32) works by them, the plain kernel token by token.  `seg_offsets` (the step's
     first row of every request, and the end of the last): tiles that were cut 8 by 8 from each request's first row are then
-    served two at a time.  Returns [T, nh*d]."""
+    served two at a time.  `spread_queries` (matrix-core sizes only, no `mix`): q comes as [T, nh, nkv, d], every head's query
+    against the key row of all groups side by side, as a caller made it.  `out_dtype` float32 (matrix-core sizes only): the result
+    in float32.  Returns [T, nh*d]."""
     _dev(q, k_cache, v_cache, block_tables, seg_of_token, positions, mix, sink)
+    if spread_queries:
+        if mix is not None or tuple(q.shape[1:]) != (nh, nkv, d) or not q.is_contiguous() or not headmix_mfma_ok(nh, nkv, d, k_cache.shape[2], q.dtype):
+            raise KernelError("queries spread over the groups are for the matrix-core kernel, [T, heads, groups, d], unmixed")
+        spread, q = q, q.view(q.shape[0], -1)
+    else:
+        spread = None
+    if out_dtype not in (None, q.dtype) and not (out_dtype == F32 and headmix_mfma_ok(nh, nkv, d, k_cache.shape[2], q.dtype)):
+        raise KernelError("a float32 result of bfloat16 operands comes from the matrix-core kernel alone")
     _i32(block_tables, "block_tables")
     _i32(seg_of_token, "seg_of_token")
     _i32(positions, "positions")
@@ -1394,11 +1404,13 @@ def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         raise KernelError(f"the heads' mixing matrix must be contiguous float32 [{nh}, {nh}]")
     if sink is not None and (sink.dtype != F32 or tuple(sink.shape) != (nh,) or not sink.is_contiguous()):
         raise KernelError(f"the denominators' extra terms must be contiguous float32 [{nh}]")
-    out = torch.empty((T, nh * d), dtype=q.dtype, device=q.device)
+    out = torch.empty((T, nh * d), dtype=out_dtype or q.dtype, device=q.device)
     if (q.dtype == BF16 and not FORCE_BASIC and USE_HEADMIX_MFMA and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0
             and _lib().ilm_attn_headmix_mfma_ok(nh, nkv, d, page)):
         # the mixing carried into the queries, then a flash attention on the matrix cores
-        if mix is None and nkv == 1 and q.stride(0) == nh * d:
+        if spread is not None:
+            qx = spread
+        elif mix is None and nkv == 1 and q.stride(0) == nh * d:
             qx = q        # one group and no mixing: the mixed queries are the queries
         else:
             qx = torch.empty((T, nh, nkv, d), dtype=BF16, device=q.device)
@@ -1437,7 +1449,7 @@ def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         _run("ilm_attn_headmix_mfma", out.data_ptr(), qx.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
              seg_of_token.data_ptr(), positions.data_ptr(), _ptr(tiles) if n_tiles else None, n_tiles, _ptr(rows), n_single,
              _ptr(sink), nh, nkv, d, page, block_tables.shape[1], out.stride(0), float(scale), int(window), _ptr(ws), nz, chunk,
-             _ptr(seg_offsets) if n_tiles else None, int(keep_first), _stream(),
+             _ptr(seg_offsets) if n_tiles else None, int(keep_first), int(out.dtype == F32), _stream(),
              label="ilm_attn_headmix_mfma (unmixed)" if mix is None and sink is None else None)
         return out
     _run("ilm_attn_headmix", out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
@@ -1451,12 +1463,14 @@ def maps_norm_rope_kvwrite(src: torch.Tensor, q_off: int, k_off: int, v_off: int
                            freq: Optional[torch.Tensor], q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
                            k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], slots: Optional[torch.Tensor],
                            heads: int, kv_heads: int, maps: int, dim: int, vdim: int, rd: int, eps: float,
-                           out_dtype: torch.dtype) -> torch.Tensor:
+                           out_dtype: torch.dtype, spread: bool = False) -> torch.Tensor:
     """From rows `src` (float32 or `out_dtype`) that hold [q: heads maps dim] at entry q_off, [k: kv_heads maps dim] at k_off
     and [v: kv_heads vdim] at v_off (k_off < 0: no keys and values in these rows): every q and k unit of `dim` entries
     RMS-normed times `q_weight` / `k_weight` [dim] (None: no norm) and its first `rd` entries turned in the pairs (i, i + rd/2)
     by position x freq[i]; k goes to the paged cache with a head's maps side by side (entry m dim + e of cache heads of d >=
-    maps dim), v to the value cache, at `slots` (None: no write).  Returns the queries [T, heads maps dim] as `out_dtype`."""
+    maps dim), v to the value cache, at `slots` (None: no write).  Returns the queries [T, heads maps dim] as `out_dtype`, or,
+    `spread`, as [T, heads maps, kv_heads, d] with zeros everywhere but at a unit's own group and map (what `headmix_attention`
+    takes as `spread_queries`)."""
     _dev(src, positions, freq, q_weight, k_weight, k_cache, v_cache, slots)
     _rows(src, "src")
     _i32(positions, "positions")
@@ -1473,19 +1487,41 @@ def maps_norm_rope_kvwrite(src: torch.Tensor, q_off: int, k_off: int, v_off: int
             raise KernelError(f"a query/key norm weight must be [{dim}]")
     page, d = 1, maps * dim
     write = k_off >= 0 and slots is not None
+    if k_cache is not None:
+        d = k_cache.shape[3]
+        page = _check_cache(k_cache, v_cache, kv_heads, d)
+    elif write or spread:
+        raise KernelError("the cache is needed for its head size")
     if write:
         _i32(slots, "slots")
         if k_cache.dtype != out_dtype or slots.numel() != T:
             raise KernelError("cache dtype or slots do not match the rows")
-        d = k_cache.shape[3]
-        page = _check_cache(k_cache, v_cache, kv_heads, d)
-    q = torch.empty((T, heads * maps * dim), dtype=out_dtype, device=src.device)
+    q = torch.empty((T, heads * maps, kv_heads, d) if spread else (T, heads * maps * dim), dtype=out_dtype, device=src.device)
     _run("ilm_maps_norm_rope_kvwrite", q.data_ptr(), src.data_ptr(), src.stride(0), int(q_off), int(k_off), int(v_off),
          positions.data_ptr(), _ptr(freq), _ptr(q_weight), _ptr(k_weight), _ptr(k_cache) if write else None,
          _ptr(v_cache) if write else None, _ptr(slots) if write else None, T, int(heads), int(kv_heads), int(maps), int(dim),
          int(vdim), int(d), int(rd), float(eps), page, _dt(src), _DT[out_dtype], _dt(q_weight) if q_weight is not None else _DT[out_dtype],
-         _stream())
+         int(bool(spread)), _stream())
     return q
+
+
+def maps_combine(a: torch.Tensor, heads: int, vdim: int, dim: int, lambda_vectors, diff: float, norm_eps: float, out_scale: float,
+                 out_dtype: torch.dtype) -> torch.Tensor:
+    """From float32 rows [T, heads x 2 x d] that hold every head's two maps' attention results: a_0 - lambda a_1 over the
+    first `vdim` entries, lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff, divided by its root mean square (norm_eps >= 0), times
+    out_scale; [T, heads vdim] as `out_dtype` (bfloat16)."""
+    _dev(a, *lambda_vectors)
+    T = a.shape[0]
+    d = a.shape[1] // (2 * heads)
+    if a.dtype != F32 or not a.is_contiguous() or a.shape[1] != heads * 2 * d or vdim > d or out_dtype != BF16:
+        raise KernelError("the maps' results are contiguous float32 rows of heads x 2 x d; the combined rows bfloat16")
+    for v in lambda_vectors:
+        if tuple(v.shape) != (dim,) or not v.is_contiguous() or v.dtype != lambda_vectors[0].dtype:
+            raise KernelError(f"the maps' weight vectors must be contiguous [{dim}] of one dtype")
+    out = torch.empty((T, heads * vdim), dtype=out_dtype, device=a.device)
+    _run("ilm_maps_combine", out.data_ptr(), a.data_ptr(), T, int(heads), int(vdim), int(d), out.stride(0), *[v.data_ptr() for v in lambda_vectors],
+         float(diff), float(norm_eps), float(out_scale), int(dim), _dt(lambda_vectors[0]), _stream())
+    return out
 
 
 def maps_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,

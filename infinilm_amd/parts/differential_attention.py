@@ -122,9 +122,22 @@ class DifferentialAttention(Mixer):
         if self.taps >= 1:
             u = kernels.causal_conv(u, self.conv_w, None, conv.pool, conv.state_in, conv.state_out, batch.seg_of_token,
                                     batch.seg_offsets, conv.state_in.numel(), "none")       # float32
-        q = kernels.maps_norm_rope_kvwrite(u, 0, self.Cq if self.own_kv else -1, self.Cq + self.Ck, batch.positions, self.freq,
-                                           self.q_norm, self.k_norm, kv.k, kv.v, kv.slots if self.own_kv else None, self.H, self.G, 2,
-                                           self.dim, self.vdim, self.rd, self.eps, self.dtype)
-        o = kernels.maps_attention(q, kv.k, kv.v, kv.block_tables, batch.seg_of_token, batch.positions, self.H, self.G, 2, self.dim,
-                                   self.vdim, self.scale, self.window, 0, None, self.lam, self.diff, self.eps, 1.0 - self.diff)
+        k_off = self.Cq if self.own_kv else -1
+        slots = kv.slots if self.own_kv else None
+        if kernels.headmix_mfma_ok(2 * self.H, self.G, self.d, kv.k.shape[2], self.dtype):
+            # bfloat16 at the matrix-core kernel's sizes: every (head, map) asks as a head of its own, with a query that is zeros
+            # outside its map's part of the key row; the two results come back in float32 and are combined and normed there
+            qx = kernels.maps_norm_rope_kvwrite(u, 0, k_off, self.Cq + self.Ck, batch.positions, self.freq, self.q_norm, self.k_norm,
+                                                kv.k, kv.v, slots, self.H, self.G, 2, self.dim, self.vdim, self.rd, self.eps, self.dtype,
+                                                spread=True)
+            a = kernels.headmix_attention(qx, kv.k, kv.v, kv.block_tables, batch.seg_of_token, batch.positions, 2 * self.H, self.G,
+                                          self.d, self.vdim, self.scale, self.window, tiles=batch.att_tiles,
+                                          single_rows=batch.att_single_rows, max_total_len=batch.max_total_len,
+                                          seg_offsets=batch.seg_offsets, spread_queries=True, out_dtype=torch.float32)
+            o = kernels.maps_combine(a, self.H, self.vdim, self.dim, self.lam, self.diff, self.eps, 1.0 - self.diff, self.dtype)
+        else:
+            q = kernels.maps_norm_rope_kvwrite(u, 0, k_off, self.Cq + self.Ck, batch.positions, self.freq, self.q_norm, self.k_norm,
+                                               kv.k, kv.v, slots, self.H, self.G, 2, self.dim, self.vdim, self.rd, self.eps, self.dtype)
+            o = kernels.maps_attention(q, kv.k, kv.v, kv.block_tables, batch.seg_of_token, batch.positions, self.H, self.G, 2, self.dim,
+                                       self.vdim, self.scale, self.window, 0, None, self.lam, self.diff, self.eps, 1.0 - self.diff)
         return self.o_proj.forward(o, allow_parts=True)
