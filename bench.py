@@ -54,7 +54,7 @@ def main() -> int:
                     help="instead of the default workload: prefill and decode throughput of another design (--design) beside MiniCPM4 "
                          "at equal layer sizes (random weights), with the time and the roofline share of every kernel")
     ap.add_argument("--design-shapes", default="1024,4096", help="widths to compare with --designs")
-    ap.add_argument("--design", default="kekevik", choices=["kekevik", "pugavik", "patadra"],
+    ap.add_argument("--design", default="kekevik", choices=["kekevik", "pugavik", "patadra", "bebuzen"],
                     help="the design that --designs puts beside MiniCPM4")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -94,7 +94,7 @@ def compare_designs(args) -> dict:
     from infinilm_amd.sampling import Sampler, SamplingParams
     from infinilm_amd.weights import fill_random_
     sys.path.insert(0, os.path.join(ROOT, "examples"))
-    from shapes import kekevik_shape, patadra_shape, pugavik_shape
+    from shapes import bebuzen_shape, kekevik_shape, patadra_shape, pugavik_shape
 
     layers = 8 if args.layers == 32 else args.layers
     T, ctx, ps = args.prefill_tokens, min(args.context, 2048), args.page_size
@@ -111,6 +111,7 @@ def compare_designs(args) -> dict:
                          "head_dim": d, "intermediate_size": 4 * width, "vocab_size": V, "max_position_embeddings": 32768,
                          "rms_norm_eps": 1e-6, "tie_word_embeddings": True},
             design: patadra_shape(width, heads, d, layers, V) if design == "patadra" else
+            bebuzen_shape(width, heads, d, kv, layers, V) if design == "bebuzen" else
             (kekevik_shape if design == "kekevik" else pugavik_shape)(width, heads, d, kv, layers, V, 6 * width)}
         rec = {}
         for name, cfg in cfgs.items():
@@ -205,17 +206,43 @@ def compare_designs(args) -> dict:
                         if us(rep_p, "ilm_stream_update"):
                             share["stream_update prefill (stream read + written, branch and gate read, rows written / HBM peak)"] = round(
                                 T * Hs * (4 + 4 + 2 + 2 + 2) / us(rep_p, "ilm_stream_update") / HBM_PEAK, 4)
+                    if name == "bebuzen":
+                        win, inner, N = 1024, 2 * Hs, 16
+                        m1 = cfg["layers"][1]["mlp"]
+                        E, top, ff = m1["router"]["experts"], m1["router"]["top"], m1["expert"]["ff"]
+                        seen, pairs = min(ctx, win), sum(min(i + 1, win) for i in range(T))
+                        for label, what in (("ilm_attn_headmix_mfma", "attention with kept first tokens"),
+                                            ("ilm_attn_headmix_mfma (unmixed)", "differential attention (two maps as heads)")):
+                            if us(rep_d, label):
+                                share[f"{what} decode (window's cache read / HBM peak)"] = round(64 * seen * kvb / us(rep_d, label) / HBM_PEAK, 4)
+                            if us(rep_p, label):
+                                share[f"{what} prefill (4 d flops a visible key and head / bf16 matrix peak)"] = round(
+                                    4.0 * d * pairs * heads / us(rep_p, label) / FLOP_PEAK["bf16"], 4)
+                        if us(rep_d, "ilm_selective_scan"):
+                            share["selective_scan decode (state read + written / HBM peak)"] = round(64 * 2 * inner * N * 4 / us(rep_d, "ilm_selective_scan") / HBM_PEAK, 4)
+                            share["selective_scan prefill (7 flops a token, channel and state entry / float32 vector peak)"] = round(
+                                7.0 * T * inner * N / us(rep_p, "ilm_selective_scan") / FLOP_PEAK["fp32"], 4)
+                        up, dn = "ilm_moe_gemm (up)", "ilm_moe_gemm (down)"
+                        if us(rep_p, up):
+                            share["experts' up product prefill (flops / bf16 matrix peak)"] = round(2.0 * T * top * ff * Hs / us(rep_p, up) / FLOP_PEAK["bf16"], 4)
+                            share["experts' down product prefill (flops / bf16 matrix peak)"] = round(2.0 * T * top * ff * Hs / us(rep_p, dn) / FLOP_PEAK["bf16"], 4)
+                            hit = min(E, 64 * top)
+                            share["experts' up product decode (weights of the experts hit read / HBM peak)"] = round(hit * ff * Hs * 2 / us(rep_d, up) / HBM_PEAK, 4)
+                            share["experts' down product decode (weights of the experts hit read / HBM peak)"] = round(hit * ff * Hs * 2 / us(rep_d, dn) / HBM_PEAK, 4)
+                        if us(rep_p, "ilm_stream_update"):
+                            share["stream_update prefill (stream read + written, branch read, rows written / HBM peak)"] = round(
+                                T * Hs * (4 + 4 + 2 + 2) / us(rep_p, "ilm_stream_update") / HBM_PEAK, 4)
                     if name == "minicpm4" and us(rep_p, "library_gemm"):
                         flops = 2.0 * T * Hs * ((heads + 2 * kv) * d + heads * d + 3 * cfg["intermediate_size"]) * layers
                         share["library products prefill, all of a step (flops / bf16 matrix peak)"] = round(
                             flops / (rep_p["library_gemm"]["total_ms"] * 1e-3 / 2) / FLOP_PEAK["bf16"], 4)
-                    if name not in ("pugavik", "patadra") and us(rep_d, "ilm_decay_scan"):
+                    if name not in ("pugavik", "patadra", "bebuzen") and us(rep_d, "ilm_decay_scan"):
                         share["decay_scan decode (state read + written / HBM peak)"] = round(64 * 2 * state / us(rep_d, "ilm_decay_scan") / HBM_PEAK, 4)
                         share["decay_scan prefill (4 dk dv flops a token and head / float32 vector peak)"] = round(
                             4.0 * T * heads * d * d / us(rep_p, "ilm_decay_scan") / FLOP_PEAK["fp32"], 4)
-                    if name not in ("pugavik", "patadra") and us(rep_d, "ilm_attn_mfma"):
+                    if name not in ("pugavik", "patadra", "bebuzen") and us(rep_d, "ilm_attn_mfma"):
                         share["attention decode (cache read / HBM peak)"] = round(64 * ctx * kvb / us(rep_d, "ilm_attn_mfma") / HBM_PEAK, 4)
-                    if name not in ("pugavik", "patadra") and us(rep_p, "ilm_attn_tile"):
+                    if name not in ("pugavik", "patadra", "bebuzen") and us(rep_p, "ilm_attn_tile"):
                         share["attention prefill (4 d flops a visible key and head / bf16 matrix peak)"] = round(
                             4.0 * T * T / 2 * heads * d / us(rep_p, "ilm_attn_tile") / FLOP_PEAK["bf16"], 4)
                     if name == "pugavik":

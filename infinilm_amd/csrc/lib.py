@@ -72,7 +72,7 @@ _SIGNATURES = {
     "ilm_maps_combine": [_P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _F, _F, _F, _I, _I, _P],
     "ilm_attn_maps": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P, _P, _P, _P, _F, _F, _F,
                       _I, _I, _P],
-    "ilm_selective_scan": [_P, _I, _P, _I, _P, _I, _P, _P, _P, _I, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+    "ilm_selective_scan": [_P, _I, _P, _I, _P, _I, _P, _P, _P, _I, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _I, _P],
     "ilm_glu_clamp": [_P, _P, _I, _I, _I, _F, _F, _I, _P],
     "ilm_head_gemm": [_P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _L, _I, _I, _P],
     "ilm_head_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _L, _P],

@@ -1569,15 +1569,19 @@ def maps_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
 
 # ---- a selective scan with a decay per channel and state entry -----------------------------------------------------------
 SELECTIVE_SCAN_MAX_STATE = 256   # most state entries a channel (ilm_selective_scan_max_state())
+SELECTIVE_SCAN_PIECE = int(os.environ.get("INFINILM_AMD_SELECTIVE_SCAN_PIECE", "64"))   # tokens a piece of a long segment (0: never cut)
+SELECTIVE_SCAN_PIECE_FROM = 128  # segments from this length on are cut into pieces that run side by side
 
 
 def selective_scan(x: torch.Tensor, raw_dt: torch.Tensor, dt_bias: torch.Tensor, B: torch.Tensor, C: torch.Tensor, z: torch.Tensor,
                    a_log: torch.Tensor, skip: torch.Tensor, pool: torch.Tensor, state_in: torch.Tensor, state_out: torch.Tensor,
-                   seg_offsets: torch.Tensor, segments: int) -> torch.Tensor:
+                   seg_offsets: torch.Tensor, segments: int, max_len: Optional[int] = None) -> torch.Tensor:
     """Per channel c and state entry n, token by token from the request's state row: dt = softplus(raw_dt + dt_bias),
     S[c, n] <- exp(-exp(a_log[c, n]) dt_c) S[c, n] + dt_c x_c B_n, y_c = sum_n S[c, n] C_n + skip_c x_c, out = y silu(z).
     x float32 [T, inner]; raw_dt, z [T, inner] and B, C [T, state] in the activations' dtype (views with dense rows; B and C of
-    one row stride); a_log float32 [inner, state], skip float32 [inner]; pool float32 [rows, inner, state].  Returns
+    one row stride); a_log float32 [inner, state], skip float32 [inner]; pool float32 [rows, inner, state].  `max_len`: a bound
+    on the segments' lengths known on the host; from SELECTIVE_SCAN_PIECE_FROM tokens on, segments are cut into pieces of
+    SELECTIVE_SCAN_PIECE tokens that run side by side (the result differs from the single pass by rounding).  Returns
     [T, inner] in the activations' dtype."""
     _dev(x, raw_dt, dt_bias, B, C, z, a_log, skip, pool, state_in, state_out, seg_offsets)
     for t, nm in ((x, "x"), (raw_dt, "raw_dt"), (B, "B"), (C, "C"), (z, "z")):
@@ -1600,10 +1604,20 @@ def selective_scan(x: torch.Tensor, raw_dt: torch.Tensor, dt_bias: torch.Tensor,
     if state_in.numel() < segments or state_out.numel() < segments or seg_offsets.numel() < segments + 1:
         raise KernelError("state rows and offsets must cover every segment")
     out = torch.empty((T, inner), dtype=dt, device=x.device)
+    piece, max_pieces, ws_state, ws_dt = 0, 0, None, None
+    if SELECTIVE_SCAN_PIECE > 0 and max_len is not None and max_len >= SELECTIVE_SCAN_PIECE_FROM:
+        piece = SELECTIVE_SCAN_PIECE
+        max_pieces = -(-int(max_len) // piece)
+        slots = T // piece + int(segments)
+        if max_pieces <= 65535:
+            ws_state = torch.empty((slots * inner * state,), dtype=F32, device=x.device)
+            ws_dt = torch.empty((slots * inner,), dtype=F32, device=x.device)
+        else:
+            piece = max_pieces = 0
     _run("ilm_selective_scan", out.data_ptr(), out.stride(0), x.data_ptr(), x.stride(0), raw_dt.data_ptr(), raw_dt.stride(0),
          dt_bias.data_ptr(), B.data_ptr(), C.data_ptr(), B.stride(0), z.data_ptr(), z.stride(0), a_log.data_ptr(), skip.data_ptr(),
-         pool.data_ptr(), state_in.data_ptr(), state_out.data_ptr(), seg_offsets.data_ptr(), int(segments), inner, state, _DT[dt],
-         _dt(dt_bias), _stream())
+         pool.data_ptr(), state_in.data_ptr(), state_out.data_ptr(), seg_offsets.data_ptr(), int(segments), inner, state, piece,
+         max_pieces, _ptr(ws_state), _ptr(ws_dt), _DT[dt], _dt(dt_bias), _stream())
     return out
 
 
@@ -1830,7 +1844,7 @@ def moe_gemm(x: torch.Tensor, w: torch.Tensor, plan: ExpertPlan, glu: bool, limi
     _run("ilm_moe_gemm", out.data_ptr(), N, x.data_ptr(), x.stride(0), plan.perm.data_ptr() if (glu or gather) else None, plan.top,
          plan.weights.data_ptr() if glu else None,
          w.data_ptr(), Nw * K, K, plan.tiles.data_ptr(), plan.n_tiles.data_ptr(), plan.max_tiles, N, K, int(bool(glu)), float(limit),
-         float(alpha), 1 if act == "relu2" else 0, _dt(x), int(MOE_FORCE_PLAIN), plan.tile_rows, int(MOE_WIDE), _stream(), label="ilm_moe_gemm (gate/up)" if glu else "ilm_moe_gemm (down)")
+         float(alpha), 1 if act == "relu2" else 0, _dt(x), int(MOE_FORCE_PLAIN), plan.tile_rows, int(MOE_WIDE), _stream(), label="ilm_moe_gemm (gate/up)" if glu else ("ilm_moe_gemm (up)" if gather else "ilm_moe_gemm (down)"))
     return out
 
 

@@ -71,5 +71,5 @@ class SelectiveScan(Mixer):
         r = self.x_proj.forward(xa)                                       # [T, dt | B | C]
         raw = self.dt_proj.forward(r[:, :R])                              # [T, inner], before bias and softplus
         y = kernels.selective_scan(xc, raw, self.dt_bias, r[:, R:R + N], r[:, R + N:], u[:, inner:], self.a_log, self.skip,
-                                   scan.pool, scan.state_in, scan.state_out, batch.seg_offsets, segments)
+                                   scan.pool, scan.state_in, scan.state_out, batch.seg_offsets, segments, max_len=batch.max_q_len)
         return self.o_proj.forward(y, allow_parts=True)

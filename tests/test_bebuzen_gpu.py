@@ -145,13 +145,19 @@ def test_norm_rotation_and_cache_write_in_maps(H, G, dim, vdim, rd, own, dtype):
 
 
 @pytest.mark.parametrize("dtype", [F32, BF])
-@pytest.mark.parametrize("inner,state", [(48, 5), (160, 20), (64, 16), (33, 1), (20, 70)])
-def test_selective_scan_carries_its_state(inner, state, dtype):
+@pytest.mark.parametrize("inner,state,lens1,lens2,pieces", [(48, 5, [7, 1, 30], [4, 9, 2], False), (160, 20, [7, 1, 30], [4, 9, 2], False),
+                                                            (64, 16, [7, 1, 30], [4, 9, 2], False), (33, 1, [7, 1, 30], [4, 9, 2], False),
+                                                            (20, 70, [7, 1, 30], [4, 9, 2], False), (64, 16, [200, 1, 64], [65, 130, 2], True),
+                                                            (40, 3, [129, 300, 5], [1, 128, 127], True), (70, 40, [140, 2, 1], [3, 190, 64], True),
+                                                            (256, 16, [7, 1, 30], [4, 9, 2], False), (300, 5, [17, 1, 33], [1, 16, 2], False),
+                                                            (512, 32, [200, 1, 64], [65, 130, 2], True), (260, 3, [129, 300, 5], [1, 128, 127], True)])
+def test_selective_scan_carries_its_state(inner, state, lens1, lens2, pieces, dtype):
     """Three requests of unequal length over two launches; the second launch starts from the rows the first left, one
-    request starts anew in a row that was used before."""
+    request starts anew in a row that was used before.  `pieces`: segments long enough to be cut into pieces of 64 tokens that
+    run side by side (lengths on either side of a piece's edge).  From 256 channels on, states of up to 32 entries take the form
+    with a thread a channel."""
     from infinilm_amd import kernels
     g = torch.Generator().manual_seed(inner + state)
-    lens1, lens2 = [7, 1, 30], [4, 9, 2]
     a_log = torch.log(0.3 + 3.0 * torch.rand(inner, state, generator=g))
     skip, bias = torch.randn(inner, generator=g), -2.0 + torch.randn(inner, generator=g)
     pool = torch.zeros((6, inner, state), device=DEV)
@@ -180,7 +186,7 @@ def test_selective_scan_carries_its_state(inner, state, dtype):
         return kernels.selective_scan(cat("x", F32), cat("raw", dtype), bias.to(dtype).to(DEV), bc[:, :state], bc[:, state:], cat("z", dtype),
                                       a_log.to(DEV), skip.to(DEV), pool, torch.tensor(rows_in, dtype=torch.int32, device=DEV),
                                       torch.tensor(rows_out, dtype=torch.int32, device=DEV), torch.tensor(offs, dtype=torch.int32, device=DEV),
-                                      len(ranges)).float().cpu()
+                                      len(ranges), max_len=max(b - a for a, b in ranges) if pieces else None).float().cpu()
 
     got1 = launch([(0, n) for n in lens1], [0, 0, 0], [1, 2, 5])
     got2 = launch([(n1, n1 + n2) for n1, n2 in zip(lens1, lens2)], [1, 2, 5], [1, 2, 5])
