@@ -120,7 +120,8 @@ def run_case(llm: LLM, case: dict, seed: int, sp_kwargs: dict) -> dict:
 def main(argv=None) -> int:
     import argparse
     extra = argparse.ArgumentParser(add_help=False)
-    extra.add_argument("--shape", choices=["8b", "0.5b", "2b", "kekevik-1024", "kekevik-4096", "pugavik-1024", "pugavik-4096"], default=None)
+    extra.add_argument("--shape", choices=["8b", "0.5b", "2b", "kekevik-1024", "kekevik-4096", "pugavik-1024", "pugavik-4096", "patadra-1024", "patadra-4096",
+                                         "bebuzen-1024", "bebuzen-4096"], default=None)
     extra.add_argument("--layers", type=int, default=0, help="with --shape: run this many layers instead of the shape's")
     extra.add_argument("--prompt-len-range", type=str, default=None, help="LO,HI: a length of its own for every request")
     ex, rest = extra.parse_known_args(sys.argv[1:] if argv is None else argv)

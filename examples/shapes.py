@@ -13,8 +13,11 @@ def _factors(n: int, seed: int):
 
 
 def shape_config(name: str, layers: int = 0) -> dict:
-    """`name`: "8b", "0.5b", "2b" (MiniCPM4 family), "kekevik-<width>", "pugavik-<width>" or "patadra-<width>" (those designs at
+    """`name`: "8b", "0.5b", "2b" (MiniCPM4 family), "kekevik-<width>", "pugavik-<width>", "patadra-<width>" or "bebuzen-<width>" (those designs at
     that width, 8 layers unless told otherwise); `layers` > 0 overrides the number of layers."""
+    if name.startswith("bebuzen-"):
+        width = int(name.split("-", 1)[1])
+        return bebuzen_shape(width, width // 128, 128, 2, layers or 8, 32768)
     if name.startswith("patadra-"):
         width = int(name.split("-")[1])
         return patadra_shape(width, width // 128, 128, layers or 8, 32768)

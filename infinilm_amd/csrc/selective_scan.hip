@@ -174,23 +174,39 @@ selective_scan_channel_kernel(T* __restrict__ out, int out_stride, const float* 
     __shared__ float stage[256 * (N + 1)];
     float S[N], A2[N];
     const int ch0 = blockIdx.x * 256, run = min(256, inner - ch0) * state;
-    {
-        const float* src = (MODE == 0 ? pool + (size_t)state_in[sgm] * inner * state : ws_state + slot * inner * state) + (size_t)ch0 * state;
-        for (int i = tid; i < run; i += 256) stage[(i / state) * (N + 1) + i % state] = MODE == 1 ? 0.f : src[i];
-        __syncthreads();
+    // every load that does not depend on another is issued before the first barrier: the state's run and A_log's (element
+    // tid + 256 j of the run), the first token's operands, the channel's constants
+    const float* src = (MODE == 0 ? pool + (size_t)state_in[sgm] * inner * state : ws_state + slot * inner * state) + (size_t)ch0 * state;
+    const float* al = a_log + (size_t)ch0 * state;
+    float s_in[N], a_in[N];
 #pragma unroll
-        for (int n = 0; n < N; ++n) S[n] = (n < state && active) ? stage[tid * (N + 1) + n] : 0.f;
-        __syncthreads();
-        const float* al = a_log + (size_t)ch0 * state;
-        for (int i = tid; i < run; i += 256) stage[(i / state) * (N + 1) + i % state] = al[i];
-        __syncthreads();
-#pragma unroll
-        for (int n = 0; n < N; ++n) A2[n] = (n < state && active) ? -expf(stage[tid * (N + 1) + n]) * 1.4426950408889634f : 0.f;
+    for (int j = 0; j < N; ++j) {
+        const int i = tid + 256 * j;
+        const int ii = i < run ? i : 0;
+        s_in[j] = MODE == 1 ? 0.f : src[ii];
+        a_in[j] = al[ii];
     }
     const float bias = to_f32(dt_bias[cc]), Dc = skip[cc];
     float dsum = 0.f;
     float xv = x[(size_t)t0 * x_stride + cc], rv = to_f32(raw[(size_t)t0 * raw_stride + cc]);
     float zv = MODE == 1 ? 0.f : to_f32(z[(size_t)t0 * z_stride + cc]);
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        const int i = tid + 256 * j;
+        if (i < run) stage[(i / state) * (N + 1) + i % state] = s_in[j];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int n = 0; n < N; ++n) S[n] = (n < state && active) ? stage[tid * (N + 1) + n] : 0.f;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        const int i = tid + 256 * j;
+        if (i < run) stage[(i / state) * (N + 1) + i % state] = a_in[j];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int n = 0; n < N; ++n) A2[n] = (n < state && active) ? -expf(stage[tid * (N + 1) + n]) * 1.4426950408889634f : 0.f;
     for (int tile = t0; tile < t1; tile += SC_TT) {
         __syncthreads();                                     // the tile before this one has been read by every thread
         for (int i = tid; i < SC_TT * N; i += 256) {
