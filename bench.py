@@ -212,7 +212,8 @@ def compare_designs(args) -> dict:
                         E, top, ff = m1["router"]["experts"], m1["router"]["top"], m1["expert"]["ff"]
                         seen, pairs = min(ctx, win), sum(min(i + 1, win) for i in range(T))
                         for label, what in (("ilm_attn_headmix_mfma", "attention with kept first tokens"),
-                                            ("ilm_attn_headmix_mfma (unmixed)", "differential attention (two maps as heads)")):
+                                            ("ilm_attn_headmix_mfma (unmixed)", "differential attention (two maps as heads)"),
+                                            ("ilm_attn_maps_mfma", "differential attention (two maps in one pass)")):
                             if us(rep_d, label):
                                 share[f"{what} decode (window's cache read / HBM peak)"] = round(64 * seen * kvb / us(rep_d, label) / HBM_PEAK, 4)
                             if us(rep_p, label):

@@ -69,6 +69,7 @@ _SIGNATURES = {
     "ilm_moe_gemm": [_P, _I, _P, _I, _P, _I, _P, _P, _L, _I, _P, _P, _I, _I, _I, _I, _F, _F, _I, _I, _I, _I, _I, _P],
     "ilm_moe_combine": [_P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _P, _I, _P],
     "ilm_maps_norm_rope_kvwrite": [_P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _P],
+    "ilm_attn_maps_mfma": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P, _P, _P, _F, _F, _F, _I, _P],
     "ilm_maps_combine": [_P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _F, _F, _F, _I, _I, _P],
     "ilm_attn_maps": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P, _P, _P, _P, _F, _F, _F,
                       _I, _I, _P],
@@ -119,6 +120,8 @@ def load(verbose: bool = True) -> ctypes.CDLL:
         fn.restype = c_int
     lib.ilm_attn_headmix_mfma_ok.restype = c_int
     lib.ilm_attn_headmix_mfma_ok.argtypes = [c_int, c_int, c_int, c_int]
+    lib.ilm_attn_maps_mfma_ok.restype = c_int
+    lib.ilm_attn_maps_mfma_ok.argtypes = [c_int, c_int, c_int, c_int, c_int, c_int]
     lib.ilm_attn_static_init.restype = c_int
     lib.ilm_attn_static_init.argtypes = []
     lib.ilm_attn_static_scratch_floats.restype = c_long

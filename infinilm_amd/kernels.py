@@ -1505,6 +1505,64 @@ def maps_norm_rope_kvwrite(src: torch.Tensor, q_off: int, k_off: int, v_off: int
     return q
 
 
+USE_MAPS_MFMA = os.environ.get("INFINILM_AMD_MAPS_MFMA", "1") == "1"   # 0: never the two-maps matrix-core kernel
+
+
+def maps_mfma_ok(heads: int, kv_heads: int, dim: int, vdim: int, d: int, page: int, dtype: torch.dtype) -> bool:
+    """Whether `maps_attention_tiles` takes these sizes (bfloat16; maps and cache heads in multiples of 32, pages of a multiple of 32)."""
+    return bool(dtype == BF16 and not FORCE_BASIC and USE_MAPS_MFMA and _lib().ilm_attn_maps_mfma_ok(heads, kv_heads, dim, vdim, d, page))
+
+
+def maps_attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                         seg_of_token: torch.Tensor, positions: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int,
+                         scale: float, window: int, lambda_vectors, diff: float, norm_eps: float, out_scale: float,
+                         tiles: Optional[torch.Tensor] = None, single_rows: Optional[torch.Tensor] = None,
+                         seg_offsets: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """`maps_attention` with two maps on the matrix cores (bfloat16, sizes of `maps_mfma_ok`), a head's two maps in one pass with
+    the combination, the norm and the scale in the kernel's epilogue.  `tiles` [n, 2] = (first row, count <= ATT_TILE_TOKENS)
+    lists runs of consecutive tokens of one request and `single_rows` the remaining rows (without them every token is served on
+    its own); `seg_offsets`: tiles cut 8 by 8 from each request's first row are then served two at a time.  An item's keys are
+    walked by one workgroup: for steps of decoded tokens alone over long windows the chunked kernel behind `headmix_attention`
+    spreads them wider.  q [T, heads 2 dim] dense; returns [T, heads vdim]."""
+    _dev(q, k_cache, v_cache, block_tables, seg_of_token, positions, tiles, single_rows, seg_offsets, *lambda_vectors)
+    _i32(block_tables, "block_tables")
+    _i32(seg_of_token, "seg_of_token")
+    _i32(positions, "positions")
+    T = q.shape[0]
+    if q.dtype != BF16 or not q.is_contiguous() or q.shape[1] != heads * 2 * dim:
+        raise KernelError(f"queries must be dense bfloat16 rows of {heads} x 2 x {dim}")
+    if k_cache.dtype != BF16 or v_cache.dtype != BF16:
+        raise KernelError("the cache must be bfloat16")
+    d = k_cache.shape[3] if k_cache.dim() == 4 else 0
+    page = _check_cache(k_cache, v_cache, kv_heads, d)
+    if not _lib().ilm_attn_maps_mfma_ok(heads, kv_heads, dim, vdim, d, page):
+        raise KernelError(f"the two-maps matrix-core kernel does not take {heads} heads in {kv_heads} groups, maps of {dim}, values of {vdim}, "
+                          f"cache heads of {d}, pages of {page}")
+    if seg_of_token.numel() != T or positions.numel() != T or block_tables.dim() != 2:
+        raise KernelError("per-token metadata does not match the number of tokens")
+    if len(lambda_vectors) != 4:
+        raise KernelError("two maps need the four vectors of their weight")
+    for v in lambda_vectors:
+        if tuple(v.shape) != (dim,) or not v.is_contiguous() or v.dtype != lambda_vectors[0].dtype:
+            raise KernelError(f"the maps' weight vectors must be contiguous [{dim}] of one dtype")
+    n_tiles, n_single, rows = 0, T, None
+    if seg_offsets is not None:
+        _i32(seg_offsets, "seg_offsets")
+    if tiles is not None and tiles.numel() > 0:
+        _i32(tiles, "tiles")
+        n_tiles, n_single = tiles.numel() // 2, 0
+        if single_rows is not None and single_rows.numel() > 0:
+            _i32(single_rows, "single_rows")
+            rows, n_single = single_rows, single_rows.numel()
+    out = torch.empty((T, heads * vdim), dtype=BF16, device=q.device)
+    _run("ilm_attn_maps_mfma", out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
+         seg_of_token.data_ptr(), positions.data_ptr(), _ptr(tiles) if n_tiles else None, n_tiles, _ptr(rows), n_single, int(heads),
+         int(kv_heads), int(dim), int(vdim), int(d), page, block_tables.shape[1], out.stride(0), float(scale), int(window),
+         _ptr(seg_offsets) if n_tiles else None, *[v.data_ptr() for v in lambda_vectors], float(diff), float(norm_eps), float(out_scale),
+         _dt(lambda_vectors[0]), _stream())
+    return out
+
+
 def maps_combine(a: torch.Tensor, heads: int, vdim: int, dim: int, lambda_vectors, diff: float, norm_eps: float, out_scale: float,
                  out_dtype: torch.dtype) -> torch.Tensor:
     """From float32 rows [T, heads x 2 x d] that hold every head's two maps' attention results: a_0 - lambda a_1 over the

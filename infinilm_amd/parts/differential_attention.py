@@ -124,7 +124,17 @@ class DifferentialAttention(Mixer):
                                     batch.seg_offsets, conv.state_in.numel(), "none")       # float32
         k_off = self.Cq if self.own_kv else -1
         slots = kv.slots if self.own_kv else None
-        if kernels.headmix_mfma_ok(2 * self.H, self.G, self.d, kv.k.shape[2], self.dtype):
+        has_runs = batch.att_tiles is not None and batch.att_tiles.numel() > 0
+        if has_runs and kernels.maps_mfma_ok(self.H, self.G, self.dim, self.vdim, self.d, kv.k.shape[2], self.dtype):
+            # bfloat16, portions of prompts, at the two-maps matrix-core kernel's sizes: both maps of a head in one pass over
+            # the keys, combined and normed in the kernel's epilogue
+            q = kernels.maps_norm_rope_kvwrite(u, 0, k_off, self.Cq + self.Ck, batch.positions, self.freq, self.q_norm, self.k_norm,
+                                               kv.k, kv.v, slots, self.H, self.G, 2, self.dim, self.vdim, self.rd, self.eps, self.dtype)
+            o = kernels.maps_attention_tiles(q, kv.k, kv.v, kv.block_tables, batch.seg_of_token, batch.positions, self.H, self.G,
+                                             self.dim, self.vdim, self.scale, self.window, self.lam, self.diff, self.eps,
+                                             1.0 - self.diff, tiles=batch.att_tiles, single_rows=batch.att_single_rows,
+                                             seg_offsets=batch.seg_offsets)
+        elif kernels.headmix_mfma_ok(2 * self.H, self.G, self.d, kv.k.shape[2], self.dtype):
             # bfloat16 at the matrix-core kernel's sizes: every (head, map) asks as a head of its own, with a query that is zeros
             # outside its map's part of the key row; the two results come back in float32 and are combined and normed there
             qx = kernels.maps_norm_rope_kvwrite(u, 0, k_off, self.Cq + self.Ck, batch.positions, self.freq, self.q_norm, self.k_norm,

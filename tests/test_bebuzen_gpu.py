@@ -334,6 +334,32 @@ def test_kept_first_tokens_on_the_matrix_cores(dtype, tmp_path):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("heads,kv,dim,vdim", [(4, 2, 64, 128), (6, 1, 32, 96), (2, 2, 32, 40), (5, 1, 32, 64)])
+def test_differential_attention_on_the_matrix_cores(dtype, heads, kv, dim, vdim, tmp_path):
+    """Maps of 32 and 64 on pages of 64 and 32 (the bfloat16 kernels' sizes; five heads leave a wave idle), window 70, 300
+    tokens: a portion from the start, a portion with history that begins inside a page, two tokens, then decoded tokens (the
+    chunked kernel); beside it a second request, so that steps hold tiles and single rows."""
+    mixer = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "diff": 0.4, "conv": 2,
+             "rot": {"base": 1000.0, "dims": dim // 2}, "mask": {"size": 70}}
+    cfg = _one_layer("attention", mixer)
+    cfg["width"] = 64
+    W = P.random_weights(cfg, 11)
+    toks, other = tokens(cfg, 300, 13), tokens(cfg, 40, 14)
+    for page in (64, 32):
+        d = str(tmp_path / f"p{page}")
+        Wr = make_dir(d, cfg, W, dtype)
+        drv = Driver(d, dtype, num_pages=-(-300 // page) + 3, page_size=page, max_requests=2)
+        drv.step([("a", toks[:150])])
+        drv.step([("a", toks[150:271]), ("b", other[:1])])
+        drv.step([("a", toks[271:273]), ("b", other[1:2])])
+        drv.step([("a", toks[273:274]), ("b", other[2:30])])
+        for i in range(274, 300):
+            drv.step([("a", [toks[i]])] + ([("b", [other[30 + i - 274]])] if 30 + i - 274 < 40 else []))
+        _close(drv.request_logits("a", 300), P.forward(cfg, Wr, toks), TOL[dtype], f"pages of {page}")
+        _close(drv.request_logits("b", 40), P.forward(cfg, Wr, other), TOL[dtype], f"second request, pages of {page}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_the_unit_term_of_the_denominator_matters(dtype, tmp_path):
     mixer = {"heads": 2, "kv_heads": 2, "dim": 8, "vdim": 8, "scale": 0.05, "mask": {"size": 30}}
     cfg = _one_layer("attention_2", mixer)
