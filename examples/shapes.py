@@ -111,15 +111,15 @@ def patadra_shape(width: int, heads: int, head_dim: int, layers: int, vocab: int
 def bebuzen_shape(width: int, heads: int, head_dim: int, kv_heads: int, layers: int, vocab: int, window: int = 1024, experts: int = 8,
                   top: int = 2) -> dict:
     """A Bebuzen configuration with the layer sizes of a transformer of this width: four layer kinds in turn (an attention with a
-    window that keeps four first tokens and a dense feed-forward of 4 x width; a differential attention with two maps of half
+    window that keeps eight first tokens and a dense feed-forward of 4 x width; a differential attention with two maps of half
     of `head_dim` each, a convolution of four taps and scaled frequencies; a selective scan over 2 x width channels with 16
     state entries each; a differential attention that reads the second layer's keys and values), the last three with `experts`
     experts of 2 x width inner units of which a token uses `top`, beside a shared expert of the same size (as many feed-forward
     weights at work for a token as in the dense layers)."""
     half = head_dim // 2
     att2 = {"heads": heads, "kv_heads": kv_heads, "dim": head_dim, "vdim": head_dim, "scale": head_dim ** -0.5,
-            "rot": {"base": 10000.0, "dims": head_dim}, "mask": {"size": window, "keep_first": 4}}
-    diff = {"heads": heads, "kv_heads": kv_heads, "dim": half, "vdim": head_dim, "scale": half ** -0.5, "diff": 0.6, "conv": 4,
+            "rot": {"base": 10000.0, "dims": head_dim}, "mask": {"size": window, "keep_first": 8}}
+    diff = {"heads": heads, "kv_heads": kv_heads, "dim": half, "vdim": head_dim, "scale": half ** -0.5, "diff": 0.5, "conv": 4,
             "rot": {"base": 500000.0, "dims": half, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}},
             "mask": {"size": window}}
     scan = {"inner": 2 * width, "state": 16, "dt_rank": max(width // 16, 1), "conv": 4}
@@ -136,4 +136,4 @@ def bebuzen_shape(width: int, heads: int, head_dim: int, kv_heads: int, layers: 
             out.append({"type": "mamba1", "mixer": dict(scan), "mlp": dict(moe)})
         else:
             out.append({"type": "attention", "mixer": dict(diff, kv_from=i - 2), "mlp": dict(moe)})
-    return {"architecture": "Bebuzen", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "residual_mult": 0.7, "layers": out}
+    return {"architecture": "Bebuzen", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.5, "layers": out}

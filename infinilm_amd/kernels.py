@@ -1665,7 +1665,9 @@ def selective_scan(x: torch.Tensor, raw_dt: torch.Tensor, dt_bias: torch.Tensor,
     piece, max_pieces, ws_state, ws_dt = 0, 0, None, None
     if SELECTIVE_SCAN_PIECE > 0 and max_len is not None and max_len >= SELECTIVE_SCAN_PIECE_FROM:
         piece = SELECTIVE_SCAN_PIECE
-        max_pieces = -(-int(max_len) // piece)
+        # (the grid holds the pieces of a segment as long as the whole step, not of the longest one now: a recorded step is
+        # replayed with other segment lengths; a piece beyond a segment's end leaves at once)
+        max_pieces = -(-T // piece)
         slots = T // piece + int(segments)
         if max_pieces <= 65535:
             ws_state = torch.empty((slots * inner * state,), dtype=F32, device=x.device)

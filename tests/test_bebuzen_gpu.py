@@ -704,6 +704,24 @@ def test_greedy_generation_through_the_entry_point(name, graph, tmp_path):
     llm.close()
 
 
+def test_recorded_steps_with_long_portions(tmp_path):
+    """Portions of up to 160 tokens (long enough for the scan's pieces) in recorded steps that are replayed with other requests'
+    portions of other lengths: greedy tokens as the plain implementation's."""
+    from infinilm_amd import LLM, SamplingParams
+    cfg = P.CONFIGS["C"]()
+    W = make_dir(str(tmp_path), cfg, P.random_weights(cfg, 78), "float32")
+    prompts = [tokens(cfg, n, 9 + n) for n in (300, 170, 129, 5, 161, 320)]
+    llm = LLM(str(tmp_path), dtype="float32", num_blocks=40, block_size=32, max_batch_size=3, chunk_size=160,
+              max_num_batched_tokens=192, enable_graph=True)
+    outs = llm.generate(prompt_token_ids=prompts, sampling_params=SamplingParams(top_k=1, max_tokens=6))
+    for prompt, out in zip(prompts, outs):
+        seq = list(prompt)
+        for _ in range(6):
+            seq.append(int(P.forward(cfg, W, seq)[-1].argmax()))
+        assert out.outputs[0].token_ids == seq[len(prompt):], f"prompt of {len(prompt)} tokens"
+    llm.close()
+
+
 def test_long_decoding(tmp_path):
     """600 decoded tokens after a prompt of 10, recorded steps, pages of 16 given back as the windows pass."""
     from infinilm_amd.engine.loading import load_model, make_runner
