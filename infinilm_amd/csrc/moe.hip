@@ -171,12 +171,15 @@ __device__ __forceinline__ uint4 moe_scale8(uint4 v, float w) {
 
 // bfloat16 on the matrix cores.  Block: 4 waves; tile: up to 64 rows of one expert x 64 outputs (GLU: 64 gate + 64 up rows of
 // W); wave w owns outputs 16 w .. 16 w + 15 for all four groups of 16 rows.  K % 8 == 0, rows 16-byte aligned.
-template <bool GLU>
+// PAIR (plain form): a workgroup takes two blocks of 64 outputs (128 rows of W), as the GLU form takes gate and up rows: twice
+// the bytes of W in flight a workgroup, which is what a step of few rows an expert (streaming W once) is bound by.
+template <bool GLU, bool PAIR = false>
 __global__ void __launch_bounds__(256)
 moe_gemm_mfma_kernel(bf16* __restrict__ out, int ld_out, const bf16* __restrict__ X, int ldx, const int* __restrict__ perm, int top,
                      const float* __restrict__ pair_w, const bf16* __restrict__ W, size_t w_expert, int ldw, const int* __restrict__ tiles,
                      const int* __restrict__ n_tiles, int N, int K, float limit, float alpha, int act) {
-    constexpr int WR = GLU ? 2 : 1;
+    constexpr int WR = (GLU || PAIR) ? 2 : 1;
+    constexpr int TNW = PAIR ? 2 * MOE_TN : MOE_TN;     // outputs a workgroup
     __shared__ __attribute__((aligned(16))) bf16 xs[MOE_TM * MOE_LD];
     __shared__ __attribute__((aligned(16))) bf16 ws[WR * MOE_TN * MOE_LD];
     __shared__ int src_row[MOE_TM];
@@ -184,7 +187,7 @@ moe_gemm_mfma_kernel(bf16* __restrict__ out, int ld_out, const bf16* __restrict_
     const int tile = blockIdx.y;
     if (tile >= *n_tiles) return;
     const int e = tiles[3 * tile], place0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
-    const int n0 = blockIdx.x * MOE_TN, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int n0 = blockIdx.x * TNW, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     if (tid < MOE_TM) {
         int row = -1;
         float w = 1.0f;
@@ -226,9 +229,9 @@ moe_gemm_mfma_kernel(bf16* __restrict__ out, int ld_out, const bf16* __restrict_
         for (int h = 0; h < WR; ++h)
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
-                const int n = n0 + lr + 32 * i;
+                const int n = n0 + lr + 32 * i + (PAIR ? h * MOE_TN : 0);
                 uint4 v = zero;
-                if (kok && n < N) v = *reinterpret_cast<const uint4*>(We + (size_t)(h * N + n) * ldw + k);
+                if (kok && n < N) v = *reinterpret_cast<const uint4*>(We + (size_t)((GLU ? h * N : 0) + n) * ldw + k);
                 wr[h * 2 + i] = v;
             }
     };
@@ -277,15 +280,17 @@ moe_gemm_mfma_kernel(bf16* __restrict__ out, int ld_out, const bf16* __restrict_
         if (m >= rows) continue;
         bf16* orow = out + (size_t)(place0 + m) * ld_out;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int n = n0 + wave * 16 + q * 4 + i;
-            if (n < N) {
-                float v = acc[0][g][i];
-                if (GLU) v = moe_glu(v, acc[WR - 1][g][i], limit, alpha);
-                else if (act == 1) { v = fmaxf(v, 0.f); v *= v; }
-                orow[n] = from_f32<bf16>(v);
+        for (int hb = 0; hb < (PAIR ? 2 : 1); ++hb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int n = n0 + hb * MOE_TN + wave * 16 + q * 4 + i;
+                if (n < N) {
+                    float v = acc[hb][g][i];
+                    if (GLU) v = moe_glu(v, acc[WR - 1][g][i], limit, alpha);
+                    else if (act == 1) { v = fmaxf(v, 0.f); v *= v; }
+                    orow[n] = from_f32<bf16>(v);
+                }
             }
-        }
     }
 }
 
@@ -553,7 +558,7 @@ extern "C" int ilm_moe_gemm(void* out, int ld_out, const void* X, int ldx, const
         // 256 rows of W a tile on demand (wide_mode 1) where the outputs fill one: a third fewer bytes a product from the caches, and
         // slower all the same at 16 experts x 256 rows, width 4,096 (622 against 545 us gate/up, 345 against 308 us down)
         const int wide_slices = glu ? (N + 127) / 128 : (N + 255) / 256;
-        const bool wide = (glu ? N >= 128 : N >= 256) && wide_mode == 1;
+        const bool wide = (glu ? N >= 128 : N >= 256) && (wide_mode & 1);
         const int n_slices = wide ? wide_slices : (glu ? (N + 63) / 64 : (N + 127) / 128);
         ILM_REQUIRE((long)max_tiles * n_slices < (1L << 30), "moe_gemm: %d tiles of %d slices are too many", max_tiles, n_slices);
         const int big = (max_tiles * n_slices + 7) / 8 * 8;      // (a multiple of 8, so every XCD's run has a workgroup for each piece)
@@ -565,6 +570,10 @@ extern "C" int ilm_moe_gemm(void* out, int ld_out, const void* X, int ldx, const
         ILM_REQUIRE(false, "moe_gemm: tiles of %d rows are the bfloat16 matrix-core kernel's alone", tile_rows);
     } else if (dtype == ILM_DTYPE_BF16 && aligned && !force_plain) {
         if (glu) moe_gemm_mfma_kernel<true><<<grid, 256, 0, stream>>>(MOE_ARGS(bf16));
+        // (measured, 64 tokens x 2 of 8 experts: 8192 x 4096 a matrix 175 -> 149 us, 4096 x 8192 204 -> 193, 16 experts of 4096 x
+        // 4096 160 -> 133; 2048 x 1024 and 1024 x 2048 27.5 -> 28.5 and 45 -> 48: only where an expert's matrix is large)
+        else if ((wide_mode & 2) && N >= 2 * MOE_TN && (long)N * K >= (1L << 23))
+            moe_gemm_mfma_kernel<false, true><<<dim3((N + 2 * MOE_TN - 1) / (2 * MOE_TN), max_tiles), 256, 0, stream>>>(MOE_ARGS(bf16));
         else moe_gemm_mfma_kernel<false><<<grid, 256, 0, stream>>>(MOE_ARGS(bf16));
     } else if (dtype == ILM_DTYPE_BF16) {
         if (glu) moe_gemm_plain_kernel<bf16, true><<<grid, 256, 0, stream>>>(MOE_ARGS(bf16));

@@ -1844,6 +1844,7 @@ MOE_TILE_ROWS = 64       # rows of one expert a workgroup of the experts' produc
 MOE_BIG_TILE_ROWS = 128  # the same for steps of many rows an expert (the bfloat16 matrix-core kernel with tiles of 128 x 128)
 MOE_BIG_MIN_ROWS = int(os.environ.get("INFINILM_AMD_MOE_BIG_MIN_ROWS", "96"))   # pairs an expert (on average) from which it runs
 MOE_FORCE_PLAIN = os.environ.get("INFINILM_AMD_MOE_PLAIN", "0") == "1"   # 1: the FMA products also in bfloat16
+MOE_PLAIN_PAIR = os.environ.get("INFINILM_AMD_MOE_PLAIN_PAIR", "1") == "1"   # the plain form's few-rows kernel takes two blocks of 64 outputs a workgroup
 MOE_WIDE = int(os.environ.get("INFINILM_AMD_MOE_WIDE", "0"))   # 1: tiles of 256 rows of W in the many-rows kernel wherever the outputs fill one (measured slower at the shapes tried)
 
 
@@ -1904,7 +1905,7 @@ def moe_gemm(x: torch.Tensor, w: torch.Tensor, plan: ExpertPlan, glu: bool, limi
     _run("ilm_moe_gemm", out.data_ptr(), N, x.data_ptr(), x.stride(0), plan.perm.data_ptr() if (glu or gather) else None, plan.top,
          plan.weights.data_ptr() if glu else None,
          w.data_ptr(), Nw * K, K, plan.tiles.data_ptr(), plan.n_tiles.data_ptr(), plan.max_tiles, N, K, int(bool(glu)), float(limit),
-         float(alpha), 1 if act == "relu2" else 0, _dt(x), int(MOE_FORCE_PLAIN), plan.tile_rows, int(MOE_WIDE), _stream(), label="ilm_moe_gemm (gate/up)" if glu else ("ilm_moe_gemm (up)" if gather else "ilm_moe_gemm (down)"))
+         float(alpha), 1 if act == "relu2" else 0, _dt(x), int(MOE_FORCE_PLAIN), plan.tile_rows, int(MOE_WIDE) | (2 if MOE_PLAIN_PAIR else 0), _stream(), label="ilm_moe_gemm (gate/up)" if glu else ("ilm_moe_gemm (up)" if gather else "ilm_moe_gemm (down)"))
     return out
 
 

@@ -203,8 +203,11 @@ def test_selective_scan_carries_its_state(inner, state, lens1, lens2, pieces, dt
 
 @pytest.mark.parametrize("dtype", [F32, BF])
 @pytest.mark.parametrize("T,width,E,top,ff,shared_ff,scale", [(1, 64, 4, 2, 24, 16, 1.5), (5, 96, 3, 1, 20, 0, 1.0), (200, 64, 8, 3, 100, 24, 2.0),
-                                                           (70, 100, 5, 5, 36, 20, 0.5), (300, 128, 2, 1, 64, 64, 1.0)])
+                                                           (70, 100, 5, 5, 36, 20, 0.5), (300, 128, 2, 1, 64, 64, 1.0),
+                                                           (9, 2048, 2, 1, 4096, 0, 1.0), (40, 2048, 3, 2, 4160, 0, 1.0)])
 def test_softmax_routed_experts_against_the_formula(T, width, E, top, ff, shared_ff, scale, dtype):
+    """(The last two shapes are large enough for the few-rows kernel that takes two blocks of outputs a workgroup; 4160 leaves
+    its last block half empty.)"""
     from infinilm_amd.parts.base import BuildContext
     from infinilm_amd.parts.moe import RoutedActivationExperts
     g = torch.Generator().manual_seed(T + E)
