@@ -208,41 +208,38 @@ moe_gemm_mfma_kernel(bf16* __restrict__ out, int ld_out, const bf16* __restrict_
     // what this thread loads a step: X rows lr, lr + 32 and W rows lr, lr + 32 (of each half), 16 bytes at k chunk lc
     const int lr = tid >> 3, lc = tid & 7;
     const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
-    uint4 xr[2], wr[WR * 2];
-    auto load = [&](int k0) {
-        const int k = k0 + lc * 8;
-        const bool kok = k < K;
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int r = src_row[lr + 32 * i];
-            uint4 v = zero;
-            if (kok && r >= 0) {
-                v = *reinterpret_cast<const uint4*>(X + (size_t)r * ldx + k);
-                // the pair's score on the rows as they are loaded: with few rows an expert this kernel streams W, and measured
-                // against the score on the float sums (as the many-rows kernel has it) it is the faster one here (192 against
-                // 235 us for 64 tokens x 2 of 16 experts at width 4,096)
-                if (GLU) v = moe_scale8(v, src_w[lr + 32 * i]);
-            }
-            xr[i] = v;
-        }
-#pragma unroll
-        for (int h = 0; h < WR; ++h)
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const int n = n0 + lr + 32 * i + (PAIR ? h * MOE_TN : 0);
-                uint4 v = zero;
-                if (kok && n < N) v = *reinterpret_cast<const uint4*>(We + (size_t)((GLU ? h * N : 0) + n) * ldw + k);
-                wr[h * 2 + i] = v;
-            }
-    };
-    auto stage = [&]() {
-#pragma unroll
-        for (int i = 0; i < 2; ++i) *reinterpret_cast<uint4*>(&xs[(lr + 32 * i) * MOE_LD + lc * 8]) = xr[i];
-#pragma unroll
-        for (int h = 0; h < WR; ++h)
-#pragma unroll
-            for (int i = 0; i < 2; ++i) *reinterpret_cast<uint4*>(&ws[(h * MOE_TN + lr + 32 * i) * MOE_LD + lc * 8]) = wr[h * 2 + i];
-    };
+    // Two sets of load registers take the k-steps in turn, so that a step's loads are in flight over two steps' products: a
+    // step of few rows an expert streams W once and waits for memory, not for the matrix cores.
+#define MOE_LOAD_SET(XR, WRG, K0)                                                                                          \
+    {                                                                                                                      \
+        const int k = (K0) + lc * 8;                                                                                       \
+        const bool kok = k < K;                                                                                            \
+        _Pragma("unroll") for (int i = 0; i < 2; ++i) {                                                                    \
+            const int r = src_row[lr + 32 * i];                                                                            \
+            uint4 v = zero;                                                                                                \
+            if (kok && r >= 0) {                                                                                           \
+                v = *reinterpret_cast<const uint4*>(X + (size_t)r * ldx + k);                                              \
+                /* the pair's score on the rows as they are loaded: with few rows an expert this kernel streams W, and */  \
+                /* measured against the score on the float sums (as the many-rows kernel has it) it is the faster one */   \
+                /* here (192 against 235 us for 64 tokens x 2 of 16 experts at width 4,096) */                             \
+                if (GLU) v = moe_scale8(v, src_w[lr + 32 * i]);                                                            \
+            }                                                                                                              \
+            XR[i] = v;                                                                                                     \
+        }                                                                                                                  \
+        _Pragma("unroll") for (int h = 0; h < WR; ++h) _Pragma("unroll") for (int i = 0; i < 2; ++i) {                      \
+            const int n = n0 + lr + 32 * i + (PAIR ? h * MOE_TN : 0);                                                      \
+            uint4 v = zero;                                                                                                \
+            if (kok && n < N) v = *reinterpret_cast<const uint4*>(We + (size_t)((GLU ? h * N : 0) + n) * ldw + k);         \
+            WRG[h * 2 + i] = v;                                                                                            \
+        }                                                                                                                  \
+    }
+#define MOE_STAGE_SET(XR, WRG)                                                                                              \
+    {                                                                                                                      \
+        _Pragma("unroll") for (int i = 0; i < 2; ++i) *reinterpret_cast<uint4*>(&xs[(lr + 32 * i) * MOE_LD + lc * 8]) = XR[i]; \
+        _Pragma("unroll") for (int h = 0; h < WR; ++h) _Pragma("unroll") for (int i = 0; i < 2; ++i)                        \
+            *reinterpret_cast<uint4*>(&ws[(h * MOE_TN + lr + 32 * i) * MOE_LD + lc * 8]) = WRG[h * 2 + i];                  \
+    }
+    uint4 xr[2], wr[WR * 2], xr2[2], wr2[WR * 2];
     f32x4 acc[WR][4];
 #pragma unroll
     for (int h = 0; h < WR; ++h)
@@ -250,12 +247,7 @@ moe_gemm_mfma_kernel(bf16* __restrict__ out, int ld_out, const bf16* __restrict_
         for (int g = 0; g < 4; ++g) acc[h][g] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int r16 = lane & 15, q = lane >> 4;
     const int groups = (rows + 15) >> 4;
-    load(0);
-    for (int k0 = 0; k0 < K; k0 += MOE_KS) {
-        __syncthreads();           // the last step's readers are done
-        stage();
-        __syncthreads();
-        if (k0 + MOE_KS < K) load(k0 + MOE_KS);
+    auto compute = [&]() {
 #pragma unroll
         for (int ks = 0; ks < MOE_KS / 32; ++ks) {
             uint4 a[WR];
@@ -272,7 +264,25 @@ moe_gemm_mfma_kernel(bf16* __restrict__ out, int ld_out, const bf16* __restrict_
                 }
             }
         }
+    };
+    MOE_LOAD_SET(xr, wr, 0)
+    MOE_LOAD_SET(xr2, wr2, MOE_KS)
+    for (int k0 = 0; k0 < K; k0 += 2 * MOE_KS) {
+        __syncthreads();           // the last step's readers are done
+        MOE_STAGE_SET(xr, wr)
+        __syncthreads();
+        if (k0 + 2 * MOE_KS < K) MOE_LOAD_SET(xr, wr, k0 + 2 * MOE_KS)
+        compute();
+        if (k0 + MOE_KS < K) {
+            __syncthreads();
+            MOE_STAGE_SET(xr2, wr2)
+            __syncthreads();
+            if (k0 + 3 * MOE_KS < K) MOE_LOAD_SET(xr2, wr2, k0 + 3 * MOE_KS)
+            compute();
+        }
     }
+#undef MOE_LOAD_SET
+#undef MOE_STAGE_SET
     // lane holds rows m = 16 g + r16 and outputs n = n0 + 16 wave + 4 q + i
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
@@ -570,8 +580,8 @@ extern "C" int ilm_moe_gemm(void* out, int ld_out, const void* X, int ldx, const
         ILM_REQUIRE(false, "moe_gemm: tiles of %d rows are the bfloat16 matrix-core kernel's alone", tile_rows);
     } else if (dtype == ILM_DTYPE_BF16 && aligned && !force_plain) {
         if (glu) moe_gemm_mfma_kernel<true><<<grid, 256, 0, stream>>>(MOE_ARGS(bf16));
-        // (measured, 64 tokens x 2 of 8 experts: 8192 x 4096 a matrix 175 -> 149 us, 4096 x 8192 204 -> 193, 16 experts of 4096 x
-        // 4096 160 -> 133; 2048 x 1024 and 1024 x 2048 27.5 -> 28.5 and 45 -> 48: only where an expert's matrix is large)
+        // (on demand, and only where an expert's matrix is large.  Measured, 64 tokens x 2 of 8 experts, with one set of load
+        // registers: 8192 x 4096 a matrix 175 -> 149 us, 4096 x 8192 204 -> 193; with two sets 132 against 135 and 129 against 138)
         else if ((wide_mode & 2) && N >= 2 * MOE_TN && (long)N * K >= (1L << 23))
             moe_gemm_mfma_kernel<false, true><<<dim3((N + 2 * MOE_TN - 1) / (2 * MOE_TN), max_tiles), 256, 0, stream>>>(MOE_ARGS(bf16));
         else moe_gemm_mfma_kernel<false><<<grid, 256, 0, stream>>>(MOE_ARGS(bf16));

@@ -1844,7 +1844,9 @@ MOE_TILE_ROWS = 64       # rows of one expert a workgroup of the experts' produc
 MOE_BIG_TILE_ROWS = 128  # the same for steps of many rows an expert (the bfloat16 matrix-core kernel with tiles of 128 x 128)
 MOE_BIG_MIN_ROWS = int(os.environ.get("INFINILM_AMD_MOE_BIG_MIN_ROWS", "96"))   # pairs an expert (on average) from which it runs
 MOE_FORCE_PLAIN = os.environ.get("INFINILM_AMD_MOE_PLAIN", "0") == "1"   # 1: the FMA products also in bfloat16
-MOE_PLAIN_PAIR = os.environ.get("INFINILM_AMD_MOE_PLAIN_PAIR", "1") == "1"   # the plain form's few-rows kernel takes two blocks of 64 outputs a workgroup
+# 1: the plain form's few-rows kernel takes two blocks of 64 outputs a workgroup for large matrices (faster while a step's loads
+# were in flight over one step's products only, 175 -> 149 us; with two sets of load registers one block is: 132 against 135 us)
+MOE_PLAIN_PAIR = os.environ.get("INFINILM_AMD_MOE_PLAIN_PAIR", "0") == "1"
 MOE_WIDE = int(os.environ.get("INFINILM_AMD_MOE_WIDE", "0"))   # 1: tiles of 256 rows of W in the many-rows kernel wherever the outputs fill one (measured slower at the shapes tried)
 
 
